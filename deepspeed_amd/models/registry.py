@@ -92,6 +92,7 @@ def _register_builtin():
     from .llama import LlamaConfig, LlamaForCausalLM
     from .lolulorn import build_from_config as build_lolulorn
     from .mixtral import MixtralConfig, MixtralForCausalLM
+    from .savovik import build_from_config as build_savovik
     hf = {"num_hidden_layers": "num_layers",
           "num_attention_heads": "num_heads",
           "num_key_value_heads": "num_kv_heads",
@@ -108,6 +109,7 @@ def _register_builtin():
         "Fizesun", lambda cfg, dtype: FizesunForCausalLM(
             FizesunConfig.from_dict(cfg), dtype))
     register_architecture("Lolulorn", build_lolulorn, wants_tensors=True)
+    register_architecture("Savovik", build_savovik)
 
 
 _register_builtin()

@@ -8,6 +8,9 @@
   ``gu`` holds gate and up side by side ([T, 2F] -> [T, F]).
 * ``glu(gu, act)``: ``act(gate) * up`` with ``act`` "silu" or "gelu_tanh"
   (``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``), same layout.
+* ``act_rows(z, act)``: a plain activation of a projection, ``act`` one of
+  "gelu_erf" (``0.5 z (1 + erf(z / sqrt 2))``), "gelu_tanh", "silu"; ``z`` may
+  be a column slice of a wider projection.
 All evaluate in fp32 and round once.
 """
 
@@ -58,3 +61,22 @@ def glu(gu, act):
     g, u = gu[..., :f].float(), gu[..., f:].float()
     a = F.silu(g) if act == "silu" else F.gelu(g, approximate="tanh")
     return (a * u).to(gu.dtype)
+
+
+ROW_ACTS = ("gelu_erf", "gelu_tanh", "silu")
+
+
+def act_rows(z, act):
+    """z [T, F] (rows contiguous, any row stride) -> act(z), contiguous."""
+    if act not in ROW_ACTS:
+        raise ValueError(f"unknown activation {act!r}")
+    if z.is_cuda and _sk().enabled():
+        return _sk().act_rows(z, ROW_ACTS.index(act))
+    zf = z.float()
+    if act == "gelu_erf":
+        y = F.gelu(zf)
+    elif act == "gelu_tanh":
+        y = F.gelu(zf, approximate="tanh")
+    else:
+        y = F.silu(zf)
+    return y.to(z.dtype)

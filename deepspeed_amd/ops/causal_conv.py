@@ -62,22 +62,29 @@ def residual_add_stats(x, delta):
     return None
 
 
-def conv_silu_ragged(x, conv_w, state, batch):
-    """Short causal convolution per channel followed by SiLU, no bias:
-    ``silu(sum_j w[:, j] * x_(t - taps + 1 + j))`` with zeros before a
-    sequence's start (the last column weighs the current token).
+def conv_silu_ragged(x, conv_w, state, batch, bias=None, out_dtype=None):
+    """Short causal convolution per channel followed by SiLU:
+    ``silu(sum_j w[:, j] * x_(t - taps + 1 + j) (+ bias))`` with zeros before
+    a sequence's start (the last column weighs the current token).
     x [T, C] (may be a column slice of a wider projection), conv_w [C, taps],
     state [slots, taps-1, C] in x's dtype: a sequence's last ``taps - 1``
     inputs, oldest first, updated in place. Sums and SiLU are fp32; returns
-    fp32 [T, C]."""
+    [T, C] fp32, or rounded once to ``out_dtype``."""
+    out_dtype = out_dtype or torch.float32
+    if x.is_cuda and _sk().enabled():
+        return _sk().conv_silu_ragged(x, conv_w, state, batch, bias,
+                                      out_dtype)
     taps = conv_w.shape[1]
     wf = conv_w.float()
-    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     at = 0
     for slot, count in zip(batch.slots, batch.counts):
         hist = torch.cat([state[slot].to(x.dtype), x[at:at + count]], 0)
         win = hist.float().unfold(0, taps, 1)          # [count, C, taps]
-        out[at:at + count] = torch.nn.functional.silu((win * wf).sum(-1))
+        acc = (win * wf).sum(-1)
+        if bias is not None:
+            acc = acc + bias.float()
+        out[at:at + count] = torch.nn.functional.silu(acc).to(out_dtype)
         if taps > 1:
             state[slot] = hist[-(taps - 1):].to(state.dtype)
         at += count

@@ -21,6 +21,13 @@ Around the scan:
   (short convolution + SiLU on q, k, v with carried tails; q and k scaled to
   unit length per head; ``beta = sigmoid(b)``;
   ``decay = exp(-exp(A_log) * softplus(a + dt_bias))``).
+* ``ssd_prep``: the scalar-decay state-space form's inputs from its fused
+  projection ``z | x | B | C | dt`` (short convolution with bias + SiLU on
+  x|B|C with carried tails; ``dt = softplus(dt + dt_bias)``;
+  ``decay = exp(-exp(A_log) * dt)``; the scan's ``v`` is ``dt * x``, its keys
+  are B and its queries C, shared by the heads of a group).
+* ``gate_group_norm``: the read-out plus the skip ``D * x``, times
+  ``silu(gate)``, then an RMS norm over equal parts of the row, times a weight.
 * ``sigmoid_pow``: ``sigmoid(z + bias) ** (1 / tau)`` for per-channel decays.
 * ``head_norm_gate``: per-head RMS norm of the read-out times a weight shared
   by the heads, times ``silu(gate)``.
@@ -123,3 +130,48 @@ def head_norm_gate(o, weight, gate, eps, out_dtype):
         return _sk().head_norm_gate(o, weight, gate, eps, out_dtype)
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
     return (y.reshape(T, H * vdim) * F.silu(gate.float())).to(out_dtype)
+
+
+def ssd_prep(proj, batch, conv_w, conv_b, conv_state, a_log, dt_bias, heads,
+             groups, state, vdim):
+    """proj [T, 2*heads*vdim + 2*groups*state + heads] =
+    z | x | B | C | dt (the z columns are left for ``gate_group_norm``).
+    conv_w [heads*vdim + 2*groups*state, taps], conv_b and conv_state
+    [slots, taps-1, same] cover the x|B|C columns.
+    Returns fp32 C [T, groups, state], B [T, groups, state],
+    v = dt * x [T, heads, vdim], x [T, heads, vdim], decay [T, heads]."""
+    T = proj.shape[0]
+    inner, gn = heads * vdim, groups * state
+    C = inner + 2 * gn
+    assert proj.shape[1] == 2 * inner + 2 * gn + heads and conv_w.shape[0] == C
+    if proj.is_cuda and _sk().enabled():
+        return _sk().ssd_prep(proj, batch, conv_w, conv_b, conv_state, a_log,
+                              dt_bias, heads, groups, state, vdim)
+    y = conv_silu_ragged(proj[:, inner:inner + C], conv_w, conv_state, batch,
+                         conv_b)
+    x = y[:, :inner].reshape(T, heads, vdim)
+    Bk = y[:, inner:inner + gn].reshape(T, groups, state)
+    Cq = y[:, inner + gn:].reshape(T, groups, state)
+    dt = F.softplus(proj[:, inner + C:].float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * dt)
+    v = dt[:, :, None] * x
+    return Cq.contiguous(), Bk.contiguous(), v, x.contiguous(), decay
+
+
+def gate_group_norm(o, x, skip, gate, weight, parts, eps, out_dtype):
+    """o, x [T, H, vdim] fp32; skip [H]; gate [T, H*vdim] pre-activation (may
+    be a column slice); weight [H*vdim]. With ``y = (o + skip_h * x) *
+    silu(gate)``, returns ``y / sqrt(mean_part(y^2) + eps) * weight`` where
+    the mean runs over each of ``parts`` equal pieces of the row, as
+    [T, H*vdim] ``out_dtype``."""
+    T, H, vdim = o.shape
+    n = H * vdim
+    assert n % parts == 0 and weight.numel() == n
+    if o.is_cuda and _sk().enabled():
+        return _sk().gate_group_norm(o, x, skip, gate, weight, parts, eps,
+                                     out_dtype)
+    y = (o + skip.float()[None, :, None] * x).reshape(T, n) \
+        * F.silu(gate.float())
+    y = y.reshape(T, parts, n // parts)
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+    return (y.reshape(T, n) * weight.float()).to(out_dtype)

@@ -210,3 +210,39 @@ def embed_rows(table, ids, scale, out_dtype=torch.float32):
     if table.is_cuda and _sk().enabled():
         return _sk().embed_rows(table, ids, scale, out_dtype)
     return (table[ids].float() * scale).to(out_dtype)
+
+
+def rms_norm_rows(x, weight, eps, out_dtype=None, index=None, one_plus=False):
+    """RMS norm with a weight per coordinate of the rows ``x[index]`` (all
+    rows without ``index``): ``x / sqrt(mean(x^2) + eps) * w``, or
+    ``* (1 + w)`` with ``one_plus`` (weights stored around zero). fp32
+    statistics and product, rounded once to ``out_dtype``."""
+    out_dtype = out_dtype or x.dtype
+    if x.is_cuda and _sk().enabled():
+        return _sk().rms_norm_rows(x.contiguous(), weight, eps, out_dtype,
+                                   index, one_plus)
+    xf = (x if index is None else x[index]).float()
+    w = weight.float() + 1.0 if one_plus else weight.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+            * w).to(out_dtype)
+
+
+def gated_add_(x, g1, y1, g2=None, y2=None, norm_weight=None, eps=1e-6,
+               out_dtype=None, one_plus=True):
+    """Sigmoid-gated residual on an fp32 stream, in place:
+    ``x += sigmoid(g1) * y1 (+ sigmoid(g2) * y2)``. ``g*`` are the gates'
+    pre-activations ([T, C], may be column slices of a wider projection),
+    ``y*`` the sublayers' results; gates, products and the sum are fp32.
+    With ``norm_weight`` the same pass also returns the RMS norm of the new
+    ``x`` (the next layer's input) in ``out_dtype``; otherwise None."""
+    assert x.dtype == torch.float32 and y1.shape == x.shape
+    if x.is_cuda and _sk().enabled():
+        return _sk().gated_add(x, g1, y1, g2, y2, norm_weight, eps,
+                               out_dtype, one_plus)
+    d = torch.sigmoid(g1.float()) * y1.float()
+    if y2 is not None:
+        d = d + torch.sigmoid(g2.float()) * y2.float()
+    x.add_(d)
+    if norm_weight is None:
+        return None
+    return rms_norm_rows(x, norm_weight, eps, out_dtype, None, one_plus)

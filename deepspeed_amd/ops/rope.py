@@ -131,3 +131,20 @@ def rope_interleaved_(x: torch.Tensor, positions: torch.Tensor,
     out = torch.stack([u * c - v * s, v * c + u * s], dim=-1)
     x[..., :rot_dims] = out.reshape(*x.shape[:-1], rot_dims).to(x.dtype)
     return x
+
+
+def rope_half_(x: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor,
+               sin: torch.Tensor, rot_dims: int) -> torch.Tensor:
+    """In-place rotary embedding pairing coordinate i with i + rot_dims/2
+    among the first ``rot_dims`` entries of the last axis; the rest pass
+    unchanged. Same operands as ``rope_interleaved_``."""
+    T = x.shape[0]
+    half = rot_dims // 2
+    shape = [T] + [1] * (x.dim() - 2) + [half]
+    c = cos[positions.long()].view(shape)
+    s = sin[positions.long()].view(shape)
+    u, v = x[..., :half].float(), x[..., half:rot_dims].float()
+    lo, hi = u * c - v * s, v * c + u * s
+    x[..., :half] = lo.to(x.dtype)
+    x[..., half:rot_dims] = hi.to(x.dtype)
+    return x
