@@ -167,8 +167,8 @@ __global__ __launch_bounds__(NT) void window_attn_k(
     const int* __restrict__ table, int maxb, int bs,
     T* __restrict__ out,       // [Ttok, H, vdim]
     float* __restrict__ part,  // [Ttok, nsplit, H, vdim + 2] when nsplit > 1
-    int H, int G, int dim, int vdim, int KC, int nsplit, float scale, int window,
-    int keep_first) {
+    int ld_out, int H, int G, int dim, int vdim, int KC, int nsplit, float scale, int window,
+    int keep_first, int chunk, float softcap, float out_scale) {
   extern __shared__ float smem[];
   const int DS = dim | 1;
   float* qs = smem;              // [WHG][dim]
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(NT) void window_attn_k(
   const int rep = H / G;
   const int row_w = G * (dim + vdim);
   const int pos = tok_pos[t];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = window > 0 ? max(0, pos - window + 1) : (chunk > 0 ? pos - pos % chunk : 0);
   const int n_keep = min(keep_first, lo);
   const int nkeys = n_keep + pos - lo + 1;
   const int* tab = table + (int64_t)tok_seq[t] * maxb;
@@ -234,6 +234,7 @@ __global__ __launch_bounds__(NT) void window_attn_k(
           const T* kr = ks + kk * DS;
           for (int c = 0; c < dim; ++c) d += qh[c] * ld(kr + c);
           d *= scale;
+          if (softcap > 0.f) d = softcap * tanhf(d / softcap);
         }
         sc[i] = d;
       }
@@ -289,11 +290,12 @@ __global__ __launch_bounds__(NT) void window_attn_k(
     for (int h = 0; h < WHG; ++h) {
       if (h < nh) {
         if (nsplit == 1) {
-          const float inv = 1.f / lrun[h];
+          const float inv = out_scale / lrun[h];
 #pragma unroll
           for (int i = 0; i < WVPT; ++i) {
             const int col = tid + i * NT;
-            if (col < vdim) st(out + ((int64_t)t * H + hbase + h) * vdim + col, acc[h][i] * inv);
+            if (col < vdim)
+              st(out + (int64_t)t * ld_out + (hbase + h) * vdim + col, acc[h][i] * inv);
           }
         } else {
           float* pp = part + (((int64_t)t * nsplit + split) * H + hbase + h) * (vdim + 2);
@@ -314,7 +316,8 @@ __global__ __launch_bounds__(NT) void window_attn_k(
 
 template <typename T>
 __global__ __launch_bounds__(NT) void window_attn_merge_k(
-    const float* __restrict__ part, T* __restrict__ out, int H, int vdim, int nsplit) {
+    const float* __restrict__ part, T* __restrict__ out, int ld_out, int H, int vdim,
+    int nsplit, float out_scale) {
   const int t = blockIdx.x, h = blockIdx.y;
   float m = -INFINITY;
   for (int s = 0; s < nsplit; ++s) {
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(NT) void window_attn_merge_k(
       const float* pp = part + (((int64_t)t * nsplit + s) * H + h) * (vdim + 2);
       if (pp[1] > 0.f) a += pp[2 + c] * expf(pp[0] - m);
     }
-    st(out + ((int64_t)t * H + h) * vdim + c, a / l);
+    st(out + (int64_t)t * ld_out + h * vdim + c, a / l * out_scale);
   }
 }
 
@@ -381,9 +384,10 @@ __global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_
     const short* __restrict__ pool,  // rows of G*dim keys then G*vdim values
     const int* __restrict__ work,    // [nwork][3] = (sequence, key/value head, first row)
     const int* __restrict__ cu, const int* __restrict__ seq_start,
-    const int* __restrict__ table, int maxb, int bs, bf16* __restrict__ out,
+    const int* __restrict__ table, int maxb, int bs, bf16* __restrict__ out, int ld_out,
     float* __restrict__ part,  // [Ttok, nsplit, H, vdim + 2] when nsplit > 1
-    int H, int G, int dim, int vdim, int nsplit, float scale, int window, int keep_first) {
+    int H, int G, int dim, int vdim, int nsplit, float scale, int window, int keep_first,
+    int chunk, float softcap, float out_scale) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   constexpr int CPT = (2 * DKT_MAX + 4 * DVB + 7) / 8;  // 16-byte chunks per thread and tile
   const int dimP = (dim + 15) & ~15;
@@ -413,8 +417,13 @@ __global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_
   const int qpos = start + j;
   const int j_lo = m0 / rep;
   const int kmax = start + min(m0 + TB_ROWS - 1, rows - 1) / rep;  // inclusive
-  const int W = window > 0 ? window : 0x7fffffff;
-  const int lo_min = window > 0 ? max(0, start + j_lo - window + 1) : 0;
+  // first key a position sees (kept first tokens aside); it never decreases
+  // along a sequence, so a tile's earliest start is its first row's
+  auto lo_of = [&](int p) -> int {
+    return window > 0 ? max(0, p - window + 1) : (chunk > 0 ? p - p % chunk : 0);
+  };
+  const int lo_q = lo_of(qpos);
+  const int lo_min = lo_of(start + j_lo);
   const int first_step = lo_min / TB_KEYS;
   const int keep_steps = keep_first > 0 ? min((keep_first - 1) / TB_KEYS + 1, first_step) : 0;
   const int nsteps = keep_steps + kmax / TB_KEYS - first_step + 1;
@@ -526,6 +535,8 @@ __global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_
   // tiles that every row sees whole)
   const int w_first = min(m0 + wid * 32, rows - 1), w_last = min(m0 + wid * 32 + 31, rows - 1);
   const int qpos_lo = start + w_first / rep, qpos_hi = start + w_last / rep;
+  const int lo_hi = lo_of(qpos_hi);
+  const float cap_inv = softcap > 0.f ? 1.f / softcap : 0.f;
 
   int64_t row_next = row_of(key0_of(v_lo));
   if (PREFETCH) {
@@ -563,19 +574,26 @@ __global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_
       }
     }
     float mx = -INFINITY;
-    if (k0 + TB_KEYS - 1 <= qpos_lo &&
-        (qpos_hi - k0 < W || k0 + TB_KEYS - 1 < keep_first)) {  // wave-uniform
+    if (softcap > 0.f) {  // uniform: s <- softcap * tanh(s / softcap)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        st[r] *= scale;
-        mx = fmaxf(mx, st[r]);
+        const float e2 = __expf(2.f * st[r] * scale * cap_inv);
+        st[r] = softcap * (1.f - 2.f / (e2 + 1.f));
       }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[r] *= scale;
+    }
+    if (k0 + TB_KEYS - 1 <= qpos_lo &&
+        (k0 >= lo_hi || k0 + TB_KEYS - 1 < keep_first)) {  // wave-uniform
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[r]);
     } else {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int key = k0 + (r & 3) + 8 * (r >> 2) + 4 * hl;
-        const bool see = key <= qpos && (qpos - key < W || key < keep_first);
-        const float sv = see ? st[r] * scale : -INFINITY;
+        const bool see = key <= qpos && (key >= lo_q || key < keep_first);
+        const float sv = see ? st[r] : -INFINITY;
         st[r] = sv;
         mx = fmaxf(mx, sv);
       }
@@ -645,8 +663,8 @@ __global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_
           if (d < vdim) pp[2 + d] = oacc[db][r];
         }
     } else {
-      const float inv = 1.f / lrun;
-      bf16* o = out + ((int64_t)t * H + h) * vdim;
+      const float inv = out_scale / lrun;
+      bf16* o = out + (int64_t)t * ld_out + h * vdim;
 #pragma unroll
       for (int db = 0; db < DVB; ++db)
 #pragma unroll
@@ -661,18 +679,21 @@ __global__ __launch_bounds__(256, (DKT_MAX <= 8 ? 2 : 1)) void window_attn_mfma_
 template <int DKT_MAX, int DVB, bool PREFETCH>
 int launch_window_attn_mfma(const void* q, const void* pool, const int* work, int nwork,
                             const int* cu, const int* seq_start, const int* table, int maxb,
-                            int bs, void* out, float* part, int Ttok, int H, int G, int dim,
-                            int vdim, int nsplit, float scale, int window, int keep_first,
+                            int bs, void* out, int ld_out, float* part, int Ttok, int H, int G,
+                            int dim, int vdim, int nsplit, float scale, int window,
+                            int keep_first, int chunk, float softcap, float out_scale,
                             hipStream_t s) {
   const int dimP = (dim + 15) & ~15;
   const size_t lds = ((size_t)TB_KEYS * (dimP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2) *
                      (PREFETCH ? 2 : 1);
   auto kern = window_attn_mfma_k<DKT_MAX, DVB, PREFETCH>;
   kern<<<dim3(nwork, nsplit), 256, lds, s>>>((const short*)q, (const short*)pool, work, cu,
-                                             seq_start, table, maxb, bs, (bf16*)out, part, H, G,
-                                             dim, vdim, nsplit, scale, window, keep_first);
+                                             seq_start, table, maxb, bs, (bf16*)out, ld_out,
+                                             part, H, G, dim, vdim, nsplit, scale, window,
+                                             keep_first, chunk, softcap, out_scale);
   if (nsplit > 1)
-    window_attn_merge_k<bf16><<<dim3(Ttok, H), NT, 0, s>>>(part, (bf16*)out, H, vdim, nsplit);
+    window_attn_merge_k<bf16><<<dim3(Ttok, H), NT, 0, s>>>(part, (bf16*)out, ld_out, H, vdim,
+                                                           nsplit, out_scale);
   return (int)hipGetLastError();
 }
 
@@ -1113,6 +1134,251 @@ __global__ __launch_bounds__(NT) void head_norm_gate_k(
   }
 }
 
+// ------------------------------------- attention prologue, per-head options
+// proj row (stride ld_proj) = [ q (H x dim) | k (G x dim) | v (G x vdim) ].
+// NORM: 0 none, 2 per head over dim with one weight of size dim shared by the
+// heads. Rotation of the first rot_dims coordinates of each head, pairing
+// (2i, 2i+1) (HALF false) or (i, i + rot_dims/2) (HALF true). v_eps >= 0:
+// every value head is divided by its root mean square. One wave per head.
+template <typename T, bool HALF>
+__global__ __launch_bounds__(NT) void attn_prep_heads_k(
+    const T* __restrict__ proj, int ld_proj, const float* __restrict__ wq,
+    const float* __restrict__ wk, const int* __restrict__ tok_pos,
+    const int* __restrict__ tok_row, const float* __restrict__ cosT,
+    const float* __restrict__ sinT, T* __restrict__ pool, T* __restrict__ q_out, int H, int G,
+    int dim, int vdim, int rot_dims, int own_kv, int norm, float eps, float v_eps) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const T* p = proj + (int64_t)t * ld_proj;
+  const int nq = H * dim, nk = G * dim, nv = G * vdim;
+  const int half = rot_dims >> 1;
+  const float* cs = cosT + (int64_t)tok_pos[t] * half;
+  const float* sn = sinT + (int64_t)tok_pos[t] * half;
+  T* row = own_kv ? pool + (int64_t)tok_row[t] * (nk + nv) : nullptr;
+  const int jobs = own_kv ? H + 2 * G : H;
+  for (int job = wid; job < jobs; job += NT / 64) {
+    if (job < H + G) {  // a query or key head
+      const bool is_q = job < H;
+      const T* in = is_q ? p + job * dim : p + nq + (job - H) * dim;
+      T* out = is_q ? q_out + (int64_t)t * nq + job * dim : row + (job - H) * dim;
+      const float* w = is_q ? wq : wk;
+      float inv = 1.f;
+      if (norm == 2) {
+        float ss = 0.f;
+        for (int c = lane; c < dim; c += 64) {
+          const float v = ld(in + c);
+          ss += v * v;
+        }
+        inv = rsqrtf(wave_sum(ss) / (float)dim + eps);
+      }
+      for (int c = lane; c < dim; c += 64) {
+        float v = ld(in + c) * inv * (norm == 2 ? w[c] : 1.f);
+        if (c < rot_dims) {
+          const int j = HALF ? (c < half ? c + half : c - half) : (c ^ 1);
+          const float o = ld(in + j) * inv * (norm == 2 ? w[j] : 1.f);
+          const int f = HALF ? (c < half ? c : c - half) : (c >> 1);
+          const bool second = HALF ? c >= half : (c & 1);
+          const float co = cs[f], si = sn[f];
+          v = second ? v * co + o * si : v * co - o * si;
+        }
+        st(out + c, v);
+      }
+    } else {  // a value head
+      const int g = job - H - G;
+      const T* in = p + nq + nk + g * vdim;
+      T* out = row + nk + g * vdim;
+      float inv = 1.f;
+      if (v_eps >= 0.f) {
+        float ss = 0.f;
+        for (int c = lane; c < vdim; c += 64) {
+          const float v = ld(in + c);
+          ss += v * v;
+        }
+        inv = rsqrtf(wave_sum(ss) / (float)vdim + v_eps);
+      }
+      for (int c = lane; c < vdim; c += 64) st(out + c, ld(in + c) * inv);
+    }
+  }
+}
+
+// ------------------------------------ short convolution + bias + SiLU, rows
+// x is a column slice (row stride ld_x) of C channels; earlier inputs come
+// from this step's rows, from the slot's tail, or are zero before position 0.
+template <typename T, typename TO>
+__global__ __launch_bounds__(NT) void conv_silu_k(
+    const T* __restrict__ x, int ld_x, const T* __restrict__ w, const float* __restrict__ bias,
+    const T* __restrict__ state, int64_t state_slot_stride, const int* __restrict__ cu,
+    const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
+    const int* __restrict__ tok_pos, TO* __restrict__ out, int C, int taps) {
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int j = t - cu[s];
+  const int pos = tok_pos[t];
+  const int tail = taps - 1;
+  const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  const T* p = x + (int64_t)t * ld_x;
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float acc = ld(w + (int64_t)c * taps + tail) * ld(p + c);
+    for (int k = 1; k < taps; ++k) {
+      if (pos - k < 0) break;
+      const float hk = k <= j ? ld(p - (int64_t)k * ld_x + c)
+                              : ld(sl + (int64_t)(tail + j - k) * C + c);
+      acc += ld(w + (int64_t)c * taps + tail - k) * hk;
+    }
+    if (bias) acc += bias[c];
+    st(out + (int64_t)t * C + c, siluf_(acc));
+  }
+}
+
+// ------------------------------------------- scalar-decay state-space prologue
+// proj row = [ z (H*P) | x (H*P) | B (G*N) | C (G*N) | dt (H) ]. One block per
+// token: convolution + bias + SiLU over the x|B|C channels,
+// dt = softplus(dt + dt_bias), decay = exp(-exp(A_log) * dt); outputs float:
+// x, v = dt * x, B, C, decay.
+template <typename T>
+__global__ __launch_bounds__(NT) void ssd_prep_k(
+    const T* __restrict__ proj, int ld_proj, const T* __restrict__ w,
+    const float* __restrict__ bias, const T* __restrict__ state, int64_t state_slot_stride,
+    const int* __restrict__ cu, const int* __restrict__ seq_slot,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    float* __restrict__ x_out, float* __restrict__ v_out, float* __restrict__ b_out,
+    float* __restrict__ c_out, float* __restrict__ decay, int H, int P, int G, int N, int taps) {
+  extern __shared__ float dts[];  // [H]
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int j = t - cu[s];
+  const int pos = tok_pos[t];
+  const int tail = taps - 1;
+  const int inner = H * P, gn = G * N;
+  const int C = inner + 2 * gn;
+  const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  const T* p = proj + (int64_t)t * ld_proj + inner;  // the convolved columns
+  for (int h = threadIdx.x; h < H; h += NT) {
+    const float dt = softplusf_(ld(p + C + h) + dt_bias[h]);
+    dts[h] = dt;
+    decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * dt);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float acc = ld(w + (int64_t)c * taps + tail) * ld(p + c);
+    for (int k = 1; k < taps; ++k) {
+      if (pos - k < 0) break;
+      const float hk = k <= j ? ld(p - (int64_t)k * ld_proj + c)
+                              : ld(sl + (int64_t)(tail + j - k) * C + c);
+      acc += ld(w + (int64_t)c * taps + tail - k) * hk;
+    }
+    const float y = siluf_(acc + bias[c]);
+    if (c < inner) {
+      x_out[(int64_t)t * inner + c] = y;
+      v_out[(int64_t)t * inner + c] = dts[c / P] * y;
+    } else if (c < inner + gn) {
+      b_out[(int64_t)t * gn + c - inner] = y;
+    } else {
+      c_out[(int64_t)t * gn + c - inner - gn] = y;
+    }
+  }
+}
+
+// y = (o + skip_h * x) * silu(gate); out = y / sqrt(mean_part(y^2) + eps) * w.
+// One block per (token, part of the row).
+template <typename T>
+__global__ __launch_bounds__(NT) void gate_group_norm_k(
+    const float* __restrict__ o, const float* __restrict__ x, const float* __restrict__ skip,
+    const T* __restrict__ gate, int ld_gate, const float* __restrict__ w, T* __restrict__ out,
+    int n, int vdim, int parts, float eps) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x, part = blockIdx.y;
+  const int len = n / parts, c0 = part * len;
+  const float* orow = o + (int64_t)t * n;
+  const float* xrow = x + (int64_t)t * n;
+  const T* grow = gate + (int64_t)t * ld_gate;
+  float ss = 0.f;
+  for (int c = c0 + threadIdx.x; c < c0 + len; c += NT) {
+    const float y = (orow[c] + skip[c / vdim] * xrow[c]) * siluf_(ld(grow + c));
+    ss += y * y;
+  }
+  const float inv = rsqrtf(block_sum(ss, red) / (float)len + eps);
+  for (int c = c0 + threadIdx.x; c < c0 + len; c += NT) {
+    const float y = (orow[c] + skip[c / vdim] * xrow[c]) * siluf_(ld(grow + c));
+    st(out + (int64_t)t * n + c, y * inv * w[c]);
+  }
+}
+
+// --------------------------------------------------------- selective scan
+// One state vector S[c, 0..N) per channel, float. SR neighbouring lanes share
+// a channel, each holding NS consecutive states in registers (N <= NS * SR); a
+// block owns NT / SR channels of one sequence and walks its tokens in order:
+//   dt = softplus(dt_pre + dt_bias); S[n] = exp(dt * A[n]) * S[n] + dt * x * B[n];
+//   y = sum_n S[n] * C[n] + D * x; out = y * silu(z) * out_scale.
+// The sum runs lane-local in a fixed order, then over the SR lanes in a fixed
+// tree, so a result does not depend on where a sequence was cut. The next
+// token's operands are loaded while the current one is computed.
+template <typename T, int NS, int SR>
+__global__ __launch_bounds__(NT) void selective_scan_k(
+    const T* __restrict__ x, int ld_x, const float* __restrict__ dt_pre,
+    const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+    const T* __restrict__ Bm, const T* __restrict__ Cm, int ld_bc,
+    const float* __restrict__ skip, const T* __restrict__ z, int ld_z,
+    float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ seq_slot,
+    T* __restrict__ out, int ld_out, int ch, int N, float out_scale) {
+  const int s = blockIdx.x;
+  const int r = threadIdx.x % SR;
+  const int c_raw = blockIdx.y * (NT / SR) + threadIdx.x / SR;
+  const bool live = c_raw < ch;
+  const int c = live ? c_raw : ch - 1;  // idle lanes shadow the last channel
+  const int n0 = r * NS;
+  float* Sg = state + ((int64_t)seq_slot[s] * ch + c) * N;
+  float S[NS], A[NS];
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const bool in = n0 + i < N;
+    S[i] = in ? Sg[n0 + i] : 0.f;
+    A[i] = in ? -expf(a_log[(int64_t)c * N + n0 + i]) : 0.f;
+  }
+  const float bias = dt_bias[c], dsk = skip[c];
+  const int t0 = cu[s], n = cu[s + 1] - t0;
+  float nb[NS], nc[NS], ndt = 0.f, nx = 0.f, nz = 0.f;
+  auto fetch = [&](int t) {
+    ndt = dt_pre[(int64_t)t * ch + c];
+    nx = ld(x + (int64_t)t * ld_x + c);
+    nz = ld(z + (int64_t)t * ld_z + c);
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const bool in = n0 + i < N;
+      nb[i] = in ? ld(Bm + (int64_t)t * ld_bc + n0 + i) : 0.f;
+      nc[i] = in ? ld(Cm + (int64_t)t * ld_bc + n0 + i) : 0.f;
+    }
+  };
+  if (n > 0) fetch(t0);
+  for (int k = 0; k < n; ++k) {
+    const float dt = softplusf_(ndt + bias), xv = nx, zv = nz;
+    float b[NS], cc[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      b[i] = nb[i];
+      cc[i] = nc[i];
+    }
+    if (k + 1 < n) fetch(t0 + k + 1);
+    const float dx = dt * xv;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      S[i] = expf(dt * A[i]) * S[i] + dx * b[i];
+      acc += S[i] * cc[i];
+    }
+#pragma unroll
+    for (int o = 1; o < SR; o <<= 1) acc += __shfl_xor(acc, o, 64);
+    if (live && r == 0)
+      st(out + (int64_t)(t0 + k) * ld_out + c, (acc + dsk * xv) * siluf_(zv) * out_scale);
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NS; ++i)
+      if (n0 + i < N) Sg[n0 + i] = S[i];
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -1144,20 +1410,24 @@ int64_t dsv_window_attn_lds(int dt, int dim, int vdim, int KC) {
 }
 
 int dsv_window_attn(const void* q, const void* pool, const int* tok_seq, const int* tok_pos,
-                    const int* table, int maxb, int bs, void* out, float* part, int dt, int Ttok,
-                    int H, int G, int dim, int vdim, int KC, int nsplit, float scale, int window,
-                    int keep_first, hipStream_t s) {
+                    const int* table, int maxb, int bs, void* out, int ld_out, float* part,
+                    int dt, int Ttok, int H, int G, int dim, int vdim, int KC, int nsplit,
+                    float scale, int window, int keep_first, int chunk, float softcap,
+                    float out_scale, hipStream_t s) {
   if (vdim > WVPT * NT || H % G || nsplit < 1 || (nsplit > 1 && !part)) return -1;
+  if ((window > 0 && chunk > 0) || ld_out < H * vdim) return -3;
   if (Ttok <= 0) return 0;
   const int64_t lds = dsv_window_attn_lds(dt, dim, vdim, KC);
   if (lds > 64 * 1024) return -2;
   dim3 grid(Ttok, G, nsplit);
   BY_DTYPE(dt, (window_attn_k<T><<<grid, NT, lds, s>>>(
                    (const T*)q, (const T*)pool, tok_seq, tok_pos, table, maxb, bs, (T*)out, part,
-                   H, G, dim, vdim, KC, nsplit, scale, window, keep_first)));
+                   ld_out, H, G, dim, vdim, KC, nsplit, scale, window, keep_first, chunk, softcap,
+                   nsplit > 1 ? 1.f : out_scale)));
   if (nsplit > 1) {
     dim3 g2(Ttok, H);
-    BY_DTYPE(dt, (window_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, H, vdim, nsplit)));
+    BY_DTYPE(dt, (window_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, ld_out, H, vdim,
+                                                           nsplit, out_scale)));
   }
   return (int)hipGetLastError();
 }
@@ -1173,15 +1443,18 @@ int dsv_window_attn_mfma_rows() { return TB_ROWS; }
 // sequence's count * (H/G) rows for that head)
 int dsv_window_attn_mfma(const void* q, const void* pool, const int* work, int nwork,
                          const int* cu, const int* seq_start, const int* table, int maxb, int bs,
-                         void* out, float* part, int Ttok, int H, int G, int dim, int vdim,
-                         int nsplit, float scale, int window, int keep_first, hipStream_t s) {
+                         void* out, int ld_out, float* part, int Ttok, int H, int G, int dim,
+                         int vdim, int nsplit, float scale, int window, int keep_first,
+                         int chunk, float softcap, float out_scale, hipStream_t s) {
   if (!dsv_window_attn_mfma_ok(dim, vdim) || H % G) return -1;
+  if ((window > 0 && chunk > 0) || ld_out < H * vdim) return -4;
   if (nsplit < 1 || (nsplit > 1 && !part)) return -3;
   if (nwork <= 0) return 0;
 #define GO(DKT, DVB, PF)                                                                        \
   return launch_window_attn_mfma<DKT, DVB, PF>(q, pool, work, nwork, cu, seq_start, table, maxb, \
-                                               bs, out, part, Ttok, H, G, dim, vdim, nsplit,     \
-                                               scale, window, keep_first, s)
+                                               bs, out, ld_out, part, Ttok, H, G, dim, vdim,     \
+                                               nsplit, scale, window, keep_first, chunk,         \
+                                               softcap, out_scale, s)
   if (dim <= 64 && vdim <= 64) GO(4, 2, true);
   if (dim <= 128 && vdim <= 128) GO(8, 4, true);
   GO(16, 8, false);
@@ -1268,6 +1541,110 @@ int dsv_head_norm_gate(const float* o, const float* w, const void* gate, int ld_
   if (Ttok <= 0) return 0;
   BY_DTYPE(dt, (head_norm_gate_k<T><<<Ttok, NT, 0, s>>>(o, w, (const T*)gate, ld_gate, (T*)out, H,
                                                         vdim, eps)));
+  return (int)hipGetLastError();
+}
+
+// norm: 0 none, 2 per head (weights of size dim); half: rotary pairing
+// (i, i + rot_dims/2) instead of (2i, 2i+1); v_eps < 0: values pass unchanged.
+int dsv_attn_prep_heads(const void* proj, int ld_proj, const float* wq, const float* wk,
+                        const int* tok_pos, const int* tok_row, const float* cosT,
+                        const float* sinT, void* pool, void* q_out, int dt, int Ttok, int H,
+                        int G, int dim, int vdim, int rot_dims, int own_kv, int norm, int half,
+                        float eps, float v_eps, hipStream_t s) {
+  if (rot_dims < 0 || (rot_dims & 1) || rot_dims > dim || H % G) return -1;
+  if ((norm != 0 && norm != 2) || (norm == 2 && (!wq || (own_kv && !wk)))) return -2;
+  if (rot_dims > 0 && (!cosT || !sinT)) return -3;
+  if (Ttok <= 0) return 0;
+  if (half)
+    BY_DTYPE(dt, (attn_prep_heads_k<T, true><<<Ttok, NT, 0, s>>>(
+                     (const T*)proj, ld_proj, wq, wk, tok_pos, tok_row, cosT, sinT, (T*)pool,
+                     (T*)q_out, H, G, dim, vdim, rot_dims, own_kv, norm, eps, v_eps)));
+  else
+    BY_DTYPE(dt, (attn_prep_heads_k<T, false><<<Ttok, NT, 0, s>>>(
+                     (const T*)proj, ld_proj, wq, wk, tok_pos, tok_row, cosT, sinT, (T*)pool,
+                     (T*)q_out, H, G, dim, vdim, rot_dims, own_kv, norm, eps, v_eps)));
+  return (int)hipGetLastError();
+}
+
+// out_dt: 0 float, otherwise the input's type
+int dsv_conv_silu(const void* x, int ld_x, const void* w, const float* bias, void* state,
+                  int64_t state_slot_stride, const int* cu, const int* seq_slot,
+                  const int* seq_start, const int* tok_seq, const int* tok_pos, void* out,
+                  int dt, int out_dt, int Ttok, int nseq, int C, int taps, hipStream_t s) {
+  if (taps < 1 || taps > MAXTAPS_SEQ || ld_x < C) return -1;
+  if (Ttok <= 0) return 0;
+  if (out_dt == 0)
+    BY_DTYPE(dt, (conv_silu_k<T, float><<<Ttok, NT, 0, s>>>(
+                     (const T*)x, ld_x, (const T*)w, bias, (const T*)state, state_slot_stride,
+                     cu, seq_slot, tok_seq, tok_pos, (float*)out, C, taps)));
+  else
+    BY_DTYPE(dt, (conv_silu_k<T, T><<<Ttok, NT, 0, s>>>(
+                     (const T*)x, ld_x, (const T*)w, bias, (const T*)state, state_slot_stride,
+                     cu, seq_slot, tok_seq, tok_pos, (T*)out, C, taps)));
+  if (taps > 1)
+    BY_DTYPE(dt, (conv_tail_shift_k<T><<<nseq, NT, 0, s>>>((const T*)x, ld_x, (T*)state,
+                                                           state_slot_stride, cu, seq_slot,
+                                                           seq_start, C, taps)));
+  return (int)hipGetLastError();
+}
+
+int dsv_ssd_prep(const void* proj, int ld_proj, const void* w, const float* bias, void* state,
+                 int64_t state_slot_stride, const int* cu, const int* seq_slot,
+                 const int* seq_start, const int* tok_seq, const int* tok_pos,
+                 const float* a_log, const float* dt_bias, float* x_out, float* v_out,
+                 float* b_out, float* c_out, float* decay, int dt, int Ttok, int nseq, int H,
+                 int P, int G, int N, int taps, hipStream_t s) {
+  if (taps < 1 || taps > MAXTAPS_SEQ || H % G || H > 16384) return -1;
+  if (ld_proj < 2 * H * P + 2 * G * N + H) return -2;
+  if (Ttok <= 0) return 0;
+  const int inner = H * P, C = inner + 2 * G * N;
+  BY_DTYPE(dt, (ssd_prep_k<T><<<Ttok, NT, H * sizeof(float), s>>>(
+                   (const T*)proj, ld_proj, (const T*)w, bias, (const T*)state,
+                   state_slot_stride, cu, seq_slot, tok_seq, tok_pos, a_log, dt_bias, x_out,
+                   v_out, b_out, c_out, decay, H, P, G, N, taps)));
+  if (taps > 1)
+    BY_DTYPE(dt, (conv_tail_shift_k<T><<<nseq, NT, 0, s>>>(
+                     (const T*)proj + inner, ld_proj, (T*)state, state_slot_stride, cu, seq_slot,
+                     seq_start, C, taps)));
+  return (int)hipGetLastError();
+}
+
+int dsv_gate_group_norm(const float* o, const float* x, const float* skip, const void* gate,
+                        int ld_gate, const float* w, void* out, int dt, int Ttok, int H, int vdim,
+                        int parts, float eps, hipStream_t s) {
+  const int n = H * vdim;
+  if (parts < 1 || n % parts || ld_gate < n) return -1;
+  if (Ttok <= 0) return 0;
+  BY_DTYPE(dt, (gate_group_norm_k<T><<<dim3(Ttok, parts), NT, 0, s>>>(
+                   o, x, skip, (const T*)gate, ld_gate, w, (T*)out, n, vdim, parts, eps)));
+  return (int)hipGetLastError();
+}
+
+// largest state size of the selective scan
+int dsv_selective_scan_max_state() { return 256; }
+
+int dsv_selective_scan(const void* x, int ld_x, const float* dt_pre, const float* dt_bias,
+                       const float* a_log, const void* Bm, const void* Cm, int ld_bc,
+                       const float* skip, const void* z, int ld_z, float* state, const int* cu,
+                       const int* seq_slot, void* out, int ld_out, int dt, int nseq, int ch,
+                       int N, float out_scale, hipStream_t s) {
+  if (N < 1 || N > dsv_selective_scan_max_state() || ch < 1) return -1;
+  if (ld_x < ch || ld_z < ch || ld_out < ch || ld_bc < N) return -2;
+  if (nseq <= 0) return 0;
+#define SSCAN(NS, SR)                                                                          \
+  do {                                                                                         \
+    dim3 grid(nseq, (ch + NT / SR - 1) / (NT / SR));                                           \
+    BY_DTYPE(dt, (selective_scan_k<T, NS, SR><<<grid, NT, 0, s>>>(                              \
+                     (const T*)x, ld_x, dt_pre, dt_bias, a_log, (const T*)Bm, (const T*)Cm,    \
+                     ld_bc, skip, (const T*)z, ld_z, state, cu, seq_slot, (T*)out, ld_out, ch, \
+                     N, out_scale)));                                                          \
+  } while (0)
+  if (N <= 16) SSCAN(4, 4);
+  else if (N <= 32) SSCAN(8, 4);
+  else if (N <= 64) SSCAN(16, 4);
+  else if (N <= 128) SSCAN(16, 8);
+  else SSCAN(16, 16);
+#undef SSCAN
   return (int)hipGetLastError();
 }
 

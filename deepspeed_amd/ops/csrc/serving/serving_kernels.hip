@@ -586,6 +586,167 @@ __global__ void topk_softmax_k(const float* __restrict__ z, int64_t* __restrict_
   for (int k = 0; k < top; ++k) w[(int64_t)t * top + k] /= sum;
 }
 
+
+// ------------------------------------------------ weighted RMS norm of rows
+// out[r] = x[idx ? idx[r] : r] / sqrt(mean(x^2) + eps) * (w or 1 + w); the
+// VEC form keeps the row in registers (C a multiple of 8, at most 8*NT*LN_G).
+template <typename TI, typename TO, bool VEC>
+__global__ __launch_bounds__(NT) void rms_norm_rows_k(
+    const TI* __restrict__ in, const int64_t* __restrict__ idx, const float* __restrict__ w,
+    TO* __restrict__ out, int C, float eps, float w_add) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  const TI* row = in + (idx ? idx[r] : r) * (int64_t)C;
+  TO* o = out + r * (int64_t)C;
+  if (VEC) {
+    float v[LN_G][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_G; ++i) {
+      const int c = (threadIdx.x + i * NT) * 8;
+      if (c < C) {
+        load8(row + c, v[i]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+      }
+    }
+    const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+#pragma unroll
+    for (int i = 0; i < LN_G; ++i) {
+      const int c = (threadIdx.x + i * NT) * 8;
+      if (c < C) {
+        float wv[8];
+        load8(w + c, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] *= inv * (wv[e] + w_add);
+        store8(o + c, v[i]);
+      }
+    }
+  } else {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < C; c += NT) {
+      const float v = ld(row + c);
+      ss += v * v;
+    }
+    const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+    for (int c = threadIdx.x; c < C; c += NT) st(o + c, ld(row + c) * inv * (w[c] + w_add));
+  }
+}
+
+// ---------------------------------------------- sigmoid-gated residual add
+// x[r] += sigmoid(g1[r]) * y1[r] (+ sigmoid(g2[r]) * y2[r]) on the float
+// stream; with a norm weight the same pass emits the RMS norm of the new row.
+// The gates are column slices of a wider projection (row stride ld_g).
+__device__ __forceinline__ float sigm(float x) { return 1.f / (1.f + expf(-x)); }
+
+template <typename T, typename TO, bool VEC>
+__global__ __launch_bounds__(NT) void gated_add_k(
+    float* __restrict__ x, const T* __restrict__ g1, const T* __restrict__ g2, int ld_g,
+    const T* __restrict__ y1, const T* __restrict__ y2, const float* __restrict__ w,
+    TO* __restrict__ h, int C, float eps, float w_add) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * C;
+  const T* a1 = g1 + r * ld_g;
+  const T* a2 = g2 ? g2 + r * ld_g : nullptr;
+  const T* b1 = y1 + r * C;
+  const T* b2 = y2 ? y2 + r * C : nullptr;
+  if (VEC) {
+    float v[LN_G][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_G; ++i) {
+      const int c = (threadIdx.x + i * NT) * 8;
+      if (c < C) {
+        float g[8], y[8];
+        load8(xr + c, v[i]);
+        load8(a1 + c, g);
+        load8(b1 + c, y);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = sigm(g[e]) * y[e];
+          g[e] = d;
+        }
+        if (a2) {
+          float g2v[8], y2v[8];
+          load8(a2 + c, g2v);
+          load8(b2 + c, y2v);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) g[e] += sigm(g2v[e]) * y2v[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          v[i][e] += g[e];
+          ss += v[i][e] * v[i][e];
+        }
+        store8(xr + c, v[i]);
+      }
+    }
+    if (!w) return;
+    const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+#pragma unroll
+    for (int i = 0; i < LN_G; ++i) {
+      const int c = (threadIdx.x + i * NT) * 8;
+      if (c < C) {
+        float wv[8];
+        load8(w + c, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] *= inv * (wv[e] + w_add);
+        store8(h + r * C + c, v[i]);
+      }
+    }
+  } else {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < C; c += NT) {
+      float d = sigm(ld(a1 + c)) * ld(b1 + c);
+      if (a2) d += sigm(ld(a2 + c)) * ld(b2 + c);
+      const float v = xr[c] + d;
+      xr[c] = v;
+      ss += v * v;
+    }
+    if (!w) return;
+    const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+    for (int c = threadIdx.x; c < C; c += NT) st(h + r * C + c, xr[c] * inv * (w[c] + w_add));
+  }
+}
+
+// -------------------------------------------------- plain row activations
+// ACT: 0 = exact GELU (erf), 1 = tanh GELU, 2 = SiLU; z is a column slice
+// with row stride ld_z, out is contiguous.
+template <int ACT>
+__device__ __forceinline__ float row_act(float z) {
+  if (ACT == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+  if (ACT == 1) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z / (1.f + expf(-z));
+}
+
+template <typename T, int ACT, bool VEC>
+__global__ void act_rows_k(const T* __restrict__ z, int ld_z, T* __restrict__ out,
+                           int64_t rows, int F) {
+  if (VEC) {
+    const int F8 = F / 8;
+    const int64_t n = rows * F8;
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x) {
+      const int64_t r = i / F8;
+      const int c = (int)(i - r * F8) * 8;
+      float v[8];
+      load8(z + r * ld_z + c, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = row_act<ACT>(v[e]);
+      store8(out + r * F + c, v);
+    }
+  } else {
+    const int64_t n = rows * F;
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x) {
+      const int64_t r = i / F;
+      const int c = (int)(i - r * F);
+      st(out + i, row_act<ACT>(ld(z + r * ld_z + c)));
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -749,6 +910,80 @@ int dsv_topk_softmax(const float* z, int64_t* idx, float* w, int Ttok, int E, in
                      hipStream_t s) {
   if (Ttok <= 0) return 0;
   topk_softmax_k<<<(Ttok + 63) / 64, 64, 0, s>>>(z, idx, w, Ttok, E, top);
+  return (int)hipGetLastError();
+}
+
+int dsv_rms_norm_rows(const void* x, int in_dt, const int64_t* idx, const float* w, void* out,
+                      int out_dt, int rows, int C, float eps, int one_plus, hipStream_t s) {
+  if (rows <= 0) return 0;
+  const float wa = one_plus ? 1.f : 0.f;
+  const bool vec = C % 8 == 0 && C <= 8 * NT * LN_G;
+#define RN(TI, TO)                                                                              \
+  do {                                                                                          \
+    if (vec)                                                                                    \
+      rms_norm_rows_k<TI, TO, true><<<rows, NT, 0, s>>>((const TI*)x, idx, w, (TO*)out, C, eps, \
+                                                        wa);                                    \
+    else                                                                                        \
+      rms_norm_rows_k<TI, TO, false><<<rows, NT, 0, s>>>((const TI*)x, idx, w, (TO*)out, C,     \
+                                                         eps, wa);                              \
+  } while (0)
+  if (in_dt == 0 && out_dt == 0) RN(float, float);
+  else if (in_dt == 0) RN(float, bf16);
+  else if (out_dt == 0) RN(bf16, float);
+  else RN(bf16, bf16);
+#undef RN
+  return (int)hipGetLastError();
+}
+
+// g1/g2: gate pre-activations with row stride ld_g (g2, y2 may be null
+// together); w null: no norm output. dt: type of the gates and results.
+int dsv_gated_add(float* x, const void* g1, const void* g2, int ld_g, const void* y1,
+                  const void* y2, const float* w, void* h, int dt, int out_dt, int rows, int C,
+                  float eps, int one_plus, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if ((g2 == nullptr) != (y2 == nullptr) || (w && !h)) return -1;
+  const float wa = one_plus ? 1.f : 0.f;
+  const bool vec = C % 8 == 0 && ld_g % 8 == 0 && C <= 8 * NT * LN_G &&
+                   ((uintptr_t)g1 % 16 == 0) && (!g2 || (uintptr_t)g2 % 16 == 0);
+#define GA(T, TO)                                                                               \
+  do {                                                                                          \
+    if (vec)                                                                                    \
+      gated_add_k<T, TO, true><<<rows, NT, 0, s>>>(x, (const T*)g1, (const T*)g2, ld_g,         \
+                                                   (const T*)y1, (const T*)y2, w, (TO*)h, C,    \
+                                                   eps, wa);                                    \
+    else                                                                                        \
+      gated_add_k<T, TO, false><<<rows, NT, 0, s>>>(x, (const T*)g1, (const T*)g2, ld_g,        \
+                                                    (const T*)y1, (const T*)y2, w, (TO*)h, C,   \
+                                                    eps, wa);                                   \
+  } while (0)
+  if (dt == 0 && out_dt == 0) GA(float, float);
+  else if (dt == 0) GA(float, bf16);
+  else if (out_dt == 0) GA(bf16, float);
+  else GA(bf16, bf16);
+#undef GA
+  return (int)hipGetLastError();
+}
+
+int dsv_act_rows(const void* z, int ld_z, void* out, int dt, int64_t rows, int F, int act,
+                 hipStream_t s) {
+  if (rows * F <= 0) return 0;
+  if (act < 0 || act > 2) return -1;
+  const bool vec = F % 8 == 0 && ld_z % 8 == 0 && (uintptr_t)z % 16 == 0;
+  const int64_t n = vec ? rows * (F / 8) : rows * F;
+  const int g = (int)((n + 255) / 256 > 262140 ? 262140 : (n + 255) / 256);
+#define AR(ACT)                                                                                 \
+  do {                                                                                          \
+    if (vec)                                                                                    \
+      BY_DTYPE(dt, (act_rows_k<T, ACT, true><<<g, 256, 0, s>>>((const T*)z, ld_z, (T*)out,      \
+                                                               rows, F)));                      \
+    else                                                                                        \
+      BY_DTYPE(dt, (act_rows_k<T, ACT, false><<<g, 256, 0, s>>>((const T*)z, ld_z, (T*)out,     \
+                                                                rows, F)));                     \
+  } while (0)
+  if (act == 0) AR(0);
+  else if (act == 1) AR(1);
+  else AR(2);
+#undef AR
   return (int)hipGetLastError();
 }
 

@@ -434,24 +434,53 @@ def _rows_ok(t):
     return t
 
 
+def _vp(t):
+    """Pointer of a view whose rows are contiguous."""
+    return ctypes.c_void_p(t.data_ptr())
+
+
 def attn_prep(proj, batch, pool, q_norm_w, k_norm_w, eps, heads, kv_heads,
-              dim, vdim, rot_dims, cos, sin, own_kv=True):
+              dim, vdim, rot_dims, cos, sin, own_kv=True, norm="whole",
+              layout="interleaved", v_unit_eps=None):
     T = proj.shape[0]
-    assert proj.is_contiguous() and proj.dtype == pool.dtype
-    assert T == batch.n_tokens and q_norm_w.numel() == heads * dim
+    _rows_ok(proj)
+    assert proj.dtype == pool.dtype and T == batch.n_tokens
     assert pool.shape[-1] == kv_heads * (dim + vdim) and pool.is_contiguous()
     assert rot_dims % 2 == 0 and rot_dims <= dim
-    assert cos.shape[1] == rot_dims // 2 and cos.shape[0] >= batch.max_ctx
-    assert cos.dtype == torch.float32 and sin.shape == cos.shape
-    if own_kv:
-        assert k_norm_w.numel() == kv_heads * dim
+    if rot_dims:
+        assert cos.shape[1] == rot_dims // 2 and cos.shape[0] >= batch.max_ctx
+        assert cos.dtype == torch.float32 and sin.shape == cos.shape
     q = torch.empty(T, heads, dim, dtype=proj.dtype, device=proj.device)
-    _check(_seq().dsv_attn_prep(
-        _p(proj), _i(proj.shape[1]), _p(_f32(q_norm_w)),
-        _p(_f32(k_norm_w) if own_kv else None), _p(batch.tok_pos),
-        _p(batch.tok_row), _p(cos), _p(sin), _p(pool), _p(q), _i(_dt(proj)),
-        _i(T), _i(heads), _i(kv_heads), _i(dim), _i(vdim), _i(rot_dims),
-        _i(1 if own_kv else 0), _f(eps), _stream()), "attn_prep")
+    if norm == "whole" and layout == "interleaved" and v_unit_eps is None:
+        assert proj.is_contiguous() and q_norm_w.numel() == heads * dim
+        if own_kv:
+            assert k_norm_w.numel() == kv_heads * dim
+        _check(_seq().dsv_attn_prep(
+            _p(proj), _i(proj.shape[1]), _p(_f32(q_norm_w)),
+            _p(_f32(k_norm_w) if own_kv else None), _p(batch.tok_pos),
+            _p(batch.tok_row), _p(cos), _p(sin), _p(pool), _p(q),
+            _i(_dt(proj)), _i(T), _i(heads), _i(kv_heads), _i(dim), _i(vdim),
+            _i(rot_dims), _i(1 if own_kv else 0), _f(eps), _stream()),
+            "attn_prep")
+        return q
+    if norm == "whole":
+        raise NotImplementedError(
+            "whole-projection norms come with interleaved rotation and plain "
+            "values only")
+    if norm == "head":
+        assert q_norm_w.numel() == dim
+        assert not own_kv or k_norm_w.numel() == dim
+    _check(_seq().dsv_attn_prep_heads(
+        _vp(proj), _i(proj.stride(0)),
+        _p(_f32(q_norm_w) if norm == "head" else None),
+        _p(_f32(k_norm_w) if norm == "head" and own_kv else None),
+        _p(batch.tok_pos), _p(batch.tok_row), _p(cos if rot_dims else None),
+        _p(sin if rot_dims else None), _p(pool), _p(q), _i(_dt(proj)), _i(T),
+        _i(heads), _i(kv_heads), _i(dim), _i(vdim), _i(rot_dims),
+        _i(1 if own_kv else 0), _i(2 if norm == "head" else 0),
+        _i(1 if layout == "half" else 0), _f(eps),
+        _f(-1.0 if v_unit_eps is None else v_unit_eps), _stream()),
+        "attn_prep_heads")
     return q
 
 
@@ -480,7 +509,8 @@ def _window_tile_work(batch, kv_heads, rep, tile_rows, device):
 
 
 def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
-                     keep_first=0, path=None):
+                     keep_first=0, path=None, chunk=0, softcap=0.0,
+                     out_scale=1.0, out=None):
     """``path`` forces "mfma" or "exact" (tests); default: the tile kernel for
     bf16 at head sizes it covers (prompt portions and, with split keys, single
     tokens), the exact kernel otherwise (fp32)."""
@@ -489,11 +519,19 @@ def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
     assert pool.shape[1] == batch.block_size and pool.is_contiguous()
     assert q.dtype == pool.dtype and H % kv_heads == 0
     assert pool.shape[-1] == kv_heads * (dim + vdim)
+    assert not (window > 0 and chunk > 0)
     lib = _seq()
     dt = _dt(q)
-    reach = batch.max_ctx if window <= 0 else \
-        min(batch.max_ctx, window + keep_first)
-    out = torch.empty(T, H, vdim, dtype=q.dtype, device=q.device)
+    reach = batch.max_ctx
+    if window > 0:
+        reach = min(reach, window + keep_first)
+    elif chunk > 0:
+        reach = min(reach, chunk + keep_first)
+    if out is None:
+        out = torch.empty(T, H * vdim, dtype=q.dtype, device=q.device)
+    assert out.shape == (T, H * vdim) and out.stride(1) == 1
+    assert out.dtype == q.dtype and out.is_cuda
+    ld_out = out.stride(0)
     mfma = q.dtype == torch.bfloat16 and \
         lib.dsv_window_attn_mfma_ok(_i(dim), _i(vdim)) == 1
     if path is None:
@@ -515,11 +553,12 @@ def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
         _check(lib.dsv_window_attn_mfma(
             _p(q), _p(pool), _p(work), _i(n), _p(batch.cu),
             _p(batch.seq_start), _p(batch.block_table),
-            _i(batch.block_table.shape[1]), _i(batch.block_size), _p(out),
-            _p(part), _i(T), _i(H), _i(kv_heads), _i(dim), _i(vdim),
-            _i(nsplit), _f(scale), _i(window), _i(keep_first), _stream()),
+            _i(batch.block_table.shape[1]), _i(batch.block_size), _vp(out),
+            _i(ld_out), _p(part), _i(T), _i(H), _i(kv_heads), _i(dim),
+            _i(vdim), _i(nsplit), _f(scale), _i(window), _i(keep_first),
+            _i(chunk), _f(softcap), _f(out_scale), _stream()),
             "window_attention(mfma)")
-        return out.view(T, H * vdim)
+        return out
     kc = 64
     while kc > 4 and lib.dsv_window_attn_lds(dt, dim, vdim, kc) > 60 * 1024:
         kc //= 2
@@ -536,10 +575,11 @@ def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
     _check(lib.dsv_window_attn(
         _p(q), _p(pool), _p(batch.tok_seq), _p(batch.tok_pos),
         _p(batch.block_table), _i(batch.block_table.shape[1]),
-        _i(batch.block_size), _p(out), _p(part), _i(dt), _i(T), _i(H),
-        _i(kv_heads), _i(dim), _i(vdim), _i(kc), _i(nsplit), _f(scale),
-        _i(window), _i(keep_first), _stream()), "window_attention")
-    return out.view(T, H * vdim)
+        _i(batch.block_size), _vp(out), _i(ld_out), _p(part), _i(dt), _i(T),
+        _i(H), _i(kv_heads), _i(dim), _i(vdim), _i(kc), _i(nsplit), _f(scale),
+        _i(window), _i(keep_first), _i(chunk), _f(softcap), _f(out_scale),
+        _stream()), "window_attention")
+    return out
 
 
 # ------------------------------------------------------ linear recurrences
@@ -623,6 +663,152 @@ def head_norm_gate(o, weight, gate, eps, out_dtype):
         _p(o), _p(_f32(weight)), ctypes.c_void_p(gate.data_ptr()),
         _i(gate.stride(0)), _p(out), _i(_DT[out_dtype]), _i(T), _i(H),
         _i(vdim), _f(eps), _stream()), "head_norm_gate")
+    return out
+
+
+# ------------------------------------- state-space prologues and epilogue
+def conv_silu_ragged(x, conv_w, state, batch, bias=None, out_dtype=None):
+    T, C = x.shape
+    taps = conv_w.shape[1]
+    out_dtype = out_dtype or torch.float32
+    _rows_ok(x)
+    assert T == batch.n_tokens and out_dtype in (torch.float32, x.dtype)
+    assert conv_w.dtype == x.dtype == state.dtype
+    assert conv_w.is_contiguous() and conv_w.shape[0] == C
+    assert state.shape[1:] == (taps - 1, C)
+    assert state.stride(2) == 1 and (taps == 1 or state.stride(1) == C)
+    out = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    _check(_seq().dsv_conv_silu(
+        _vp(x), _i(x.stride(0)), _p(conv_w),
+        _p(None if bias is None else _f32(bias)), _vp(state),
+        _l(state.stride(0)), _p(batch.cu), _p(batch.seq_slot),
+        _p(batch.seq_start), _p(batch.tok_seq), _p(batch.tok_pos), _p(out),
+        _i(_dt(x)), _i(0 if out_dtype == torch.float32 else 1), _i(T),
+        _i(batch.n_seqs), _i(C), _i(taps), _stream()), "conv_silu")
+    return out
+
+
+def ssd_prep(proj, batch, conv_w, conv_b, conv_state, a_log, dt_bias, heads,
+             groups, state, vdim):
+    T = proj.shape[0]
+    taps = conv_w.shape[1]
+    inner, gn = heads * vdim, groups * state
+    C = inner + 2 * gn
+    _rows_ok(proj)
+    assert T == batch.n_tokens and proj.shape[1] == 2 * inner + 2 * gn + heads
+    assert conv_w.dtype == proj.dtype == conv_state.dtype
+    assert conv_w.is_contiguous() and conv_w.shape[0] == C
+    assert conv_b.numel() == C and a_log.numel() == heads
+    assert dt_bias.numel() == heads
+    assert conv_state.shape[1:] == (taps - 1, C)
+    assert conv_state.stride(2) == 1 and (taps == 1
+                                          or conv_state.stride(1) == C)
+    f32 = dict(dtype=torch.float32, device=proj.device)
+    x = torch.empty(T, heads, vdim, **f32)
+    v = torch.empty(T, heads, vdim, **f32)
+    Bk = torch.empty(T, groups, state, **f32)
+    Cq = torch.empty(T, groups, state, **f32)
+    decay = torch.empty(T, heads, **f32)
+    _check(_seq().dsv_ssd_prep(
+        _vp(proj), _i(proj.stride(0)), _p(conv_w), _p(_f32(conv_b)),
+        _vp(conv_state), _l(conv_state.stride(0)), _p(batch.cu),
+        _p(batch.seq_slot), _p(batch.seq_start), _p(batch.tok_seq),
+        _p(batch.tok_pos), _p(_f32(a_log)), _p(_f32(dt_bias)), _p(x), _p(v),
+        _p(Bk), _p(Cq), _p(decay), _i(_dt(proj)), _i(T), _i(batch.n_seqs),
+        _i(heads), _i(vdim), _i(groups), _i(state), _i(taps), _stream()),
+        "ssd_prep")
+    return Cq, Bk, v, x, decay
+
+
+def gate_group_norm(o, x, skip, gate, weight, parts, eps, out_dtype):
+    T, H, vdim = o.shape
+    n = H * vdim
+    assert o.dtype == torch.float32 and o.is_contiguous()
+    assert x.dtype == torch.float32 and x.is_contiguous() and x.shape == o.shape
+    assert skip.numel() == H and weight.numel() == n and n % parts == 0
+    assert gate.shape == (T, n) and gate.dtype == out_dtype
+    _rows_ok(gate)
+    out = torch.empty(T, n, dtype=out_dtype, device=o.device)
+    _check(_seq().dsv_gate_group_norm(
+        _p(o), _p(x), _p(_f32(skip)), _vp(gate), _i(gate.stride(0)),
+        _p(_f32(weight)), _p(out), _i(_DT[out_dtype]), _i(T), _i(H), _i(vdim),
+        _i(parts), _f(eps), _stream()), "gate_group_norm")
+    return out
+
+
+def selective_scan(x, dt_pre, dt_bias, a_log, B, C, skip, z, state, batch,
+                   out_scale, out):
+    T, ch = x.shape
+    n = a_log.shape[1]
+    for t in (x, B, C, z, out):
+        _rows_ok(t)
+    assert x.dtype == B.dtype == C.dtype == z.dtype == out.dtype
+    assert B.stride(0) == C.stride(0) and T == batch.n_tokens
+    assert dt_pre.is_contiguous() and dt_pre.dtype == torch.float32
+    assert state.dtype == torch.float32 and state.is_contiguous()
+    assert state.shape[1:] == (ch, n) and a_log.shape == (ch, n)
+    assert dt_bias.numel() == ch and skip.numel() == ch
+    lib = _seq()
+    if n > lib.dsv_selective_scan_max_state():
+        raise ValueError("selective scan: state size beyond the kernel's")
+    _check(lib.dsv_selective_scan(
+        _vp(x), _i(x.stride(0)), _p(dt_pre), _p(_f32(dt_bias)),
+        _p(_f32(a_log).contiguous()), _vp(B), _vp(C), _i(B.stride(0)),
+        _p(_f32(skip)), _vp(z), _i(z.stride(0)), _p(state), _p(batch.cu),
+        _p(batch.seq_slot), _vp(out), _i(out.stride(0)), _i(_dt(x)),
+        _i(batch.n_seqs), _i(ch), _i(n), _f(out_scale), _stream()),
+        "selective_scan")
+    return out
+
+
+# --------------------------------------- weighted RMS norm, gated residual
+def rms_norm_rows(x, weight, eps, out_dtype, index=None, one_plus=False):
+    rows = x.shape[0] if index is None else index.numel()
+    C = x.shape[1]
+    assert weight.numel() == C and x.is_contiguous()
+    out = torch.empty(rows, C, dtype=out_dtype, device=x.device)
+    if index is not None:
+        index = index.to(torch.int64).contiguous()
+    _check(load().dsv_rms_norm_rows(
+        _p(x), _i(_dt(x)), _p(index), _p(_f32(weight)), _p(out),
+        _i(_DT[out_dtype]), _i(rows), _i(C), _f(eps), _i(1 if one_plus else 0),
+        _stream()), "rms_norm_rows")
+    return out
+
+
+def gated_add(x, g1, y1, g2, y2, norm_weight, eps, out_dtype, one_plus):
+    T, C = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert g1.shape == (T, C) and y1.shape == (T, C)
+    _rows_ok(g1)
+    y1 = y1.contiguous()
+    assert g1.dtype == y1.dtype
+    if y2 is not None:
+        _rows_ok(g2)
+        y2 = y2.contiguous()
+        assert g2.shape == (T, C) and y2.shape == (T, C)
+        assert g2.dtype == y2.dtype == y1.dtype
+        assert g2.stride(0) == g1.stride(0)
+    h = None
+    if norm_weight is not None:
+        out_dtype = out_dtype or torch.float32
+        assert norm_weight.numel() == C
+        h = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    _check(load().dsv_gated_add(
+        _p(x), _vp(g1), _p(None) if y2 is None else _vp(g2),
+        _i(g1.stride(0)), _p(y1), _p(y2),
+        _p(None if norm_weight is None else _f32(norm_weight)), _p(h),
+        _i(_dt(y1)), _i(0 if h is None else _DT[h.dtype]), _i(T), _i(C),
+        _f(eps), _i(1 if one_plus else 0), _stream()), "gated_add")
+    return h
+
+
+def act_rows(z, act):
+    T, F = z.shape
+    _rows_ok(z)
+    out = torch.empty(T, F, dtype=z.dtype, device=z.device)
+    _check(load().dsv_act_rows(_vp(z), _i(z.stride(0)), _p(out), _i(_dt(z)),
+                               _l(T), _i(F), _i(act), _stream()), "act_rows")
     return out
 
 
