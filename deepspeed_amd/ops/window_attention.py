@@ -47,7 +47,7 @@ def _qk_norm(x, w, eps, norm, n_heads, dim):
     xf = x.float().reshape(T, n_heads, dim)
     if norm == "head":
         return _rms_all(xf, w, eps)
-    return xf
+    return xf.clone()           # rotated in place: never the caller's rows
 
 
 def attn_prep(proj, batch, pool, q_norm_w, k_norm_w, eps, heads, kv_heads,
