@@ -12,6 +12,11 @@ Run through ``python bench.py --serving fizesun``.
 ``--serving lolulorn`` does the same for Lolulorn (one block of gla /
 attention / attention on borrowed rows / delta layers, dense and routed
 feed-forwards) beside Llama, with Fizesun's throughput for the ragged path.
+
+``--serving savovik`` runs Savovik (one block of mamba2 / capped windowed
+attention / chunked attention beside a selective scan / mamba2 on the first
+layer's weights) beside Lolulorn, its closest sibling on the ragged path, and
+Llama; every Savovik kernel is timed next to the like Lolulorn kernel.
 """
 
 import json
@@ -493,6 +498,296 @@ def run_lolulorn(sizes=("s", "m", "l"), kernels=True):
     return report
 
 
+
+# -------------------------------------------------------------- Savovik
+def savovik_config(z, vocab=32000):
+    """One block [mamba2, attention, parallel, mamba2 on the first layer's
+    weights] repeated to ``layers``: state-space heads of 64 with a state of
+    128 (inner = 2 x width); attention heads of 128, 4 query heads per
+    key/value head, window 1024, scores capped at 30; the parallel mixer's
+    attention confined to chunks of 1024 beside a selective scan over
+    ``width`` channels with 16 states each."""
+    H, W = z["heads"], z["width"]
+    att = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128,
+           "scale": 128 ** -0.5, "softcap": 30.0, "mask": {"size": 1024},
+           "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 2.0}}}
+    left = {"heads": max(1, H // 2), "kv_heads": max(1, H // 8), "dim": 128,
+            "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+            "rot": {"base": 500000.0, "dims": 64,
+                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                "original": 8192}}}
+    right = {"inner": W, "state": 16, "dt_rank": max(1, W // 16), "conv": 4}
+    m2 = {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8,
+          "norm_groups": 8, "conv": 4}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    layers = []
+    for i in range(z["layers"]):
+        kind = i % 4
+        if kind in (0, 3):
+            spec = {"type": "mamba2", "mixer": m2, "mlp": dense}
+            if kind == 3:
+                spec["weights_of"] = i - 3
+            layers.append(spec)
+        elif kind == 1:
+            layers.append({"type": "attention", "mixer": att, "mlp": dense})
+        else:
+            layers.append({"type": "parallel", "mlp": dense, "mixer": {
+                "left": left, "right": right, "left_scale": 1.0,
+                "right_scale": 1.0}})
+    return {"architecture": "Savovik", "vocab": vocab, "width": W,
+            "norm": {"eps": 1e-6}, "layers": layers}
+
+
+@torch.no_grad()
+def _savovik_kernel_rows(z, dev):
+    """Every Savovik kernel at this size, each followed by the like kernel of
+    the Lolulorn path ("like" names it; rows with an empty "like" are the
+    siblings themselves)."""
+    from ..ops import serving_kernels as sk
+    from ..ops.rope import rope_tables
+    from .state_cache import PagedStateCache
+    bf = torch.bfloat16
+    B, S, W, H = z["batch"], z["seq"], z["width"], z["heads"]
+    F = z["ff"]
+    G, d, dv = max(1, H // 4), 128, 128
+    T = B * S
+    out = []
+
+    def row(name, like, fn, nbytes, flops=0.0, iters=5):
+        t = _timed(fn, 2, iters)
+        bound = max(nbytes / HBM_BW, flops / MFMA_BF16)
+        out.append({"kernel": name, "like": like, "us": 1e6 * t,
+                    "bound_us": 1e6 * bound, "distance": t / bound})
+
+    # ---- gated residual (+ next norm) against the post-norm residual
+    x32 = torch.randn(T, W, device=dev)
+    side = torch.randn(T, 2 * W + 64, device=dev).to(bf)
+    y1 = (torch.randn(T, W, device=dev) * 0.01).to(bf)
+    y2 = (torch.randn(T, W, device=dev) * 0.01).to(bf)
+    wn = torch.zeros(W, device=dev)
+    row("gated_add (fp32 stream += 2 gated bf16 results, bf16 norm out)",
+        "layer_norm_add",
+        lambda: sk.gated_add(x32, side[:, :W], y1, side[:, W:2 * W], y2, wn,
+                             1e-6, bf, True), T * W * 18)
+    bn = torch.zeros(W, device=dev)
+    row("layer_norm_add (lolulorn)", "",
+        lambda: sk.layer_norm_add(x32, y1, wn + 1, bn, 1e-6, bf), T * W * 12)
+    # ---- attention prologues
+    cache = PagedStateCache([G * (d + dv)], {}, B, B * (S + 64), dtype=bf,
+                            device=dev)
+    batch = cache.begin_ragged(list(range(B)), [S] * B)
+    cos, sin = rope_tables(64, cache.max_seq, 10000.0, device=dev, scaling=2.0)
+    proj = torch.randn(T, (H + 2 * G) * d, device=dev).to(bf)
+    hw = torch.ones(d, device=dev)
+    nb = T * (H + 2 * G) * d * 4
+    row("attn_prep: rotate-half, unit values, cache write", "attn_prep",
+        lambda: sk.attn_prep(proj, batch, cache.pools[0], None, None, 1e-6, H,
+                             G, d, dv, 64, cos, sin, True, None, "half",
+                             1e-6), nb)
+    row("attn_prep: per-head q/k norm, interleaved rotary, cache write",
+        "attn_prep",
+        lambda: sk.attn_prep(proj, batch, cache.pools[0], hw, hw, 1e-6, H, G,
+                             d, dv, 64, cos, sin, True, "head", "interleaved",
+                             None), nb)
+    qw, kw = torch.ones(H * d, device=dev), torch.ones(G * d, device=dev)
+    row("attn_prep (lolulorn: whole-projection norms)", "",
+        lambda: sk.attn_prep(proj, batch, cache.pools[0], qw, kw, 1e-6, H, G,
+                             d, dv, 64, cos, sin, True), nb)
+    # ---- prefill attention
+    q = sk.attn_prep(proj, batch, cache.pools[0], hw, hw, 1e-6, H, G, d, dv,
+                     64, cos, sin, True, "head", "interleaved", None)
+    win = 1024
+    seen_w = sum(min(i + 1, win) for i in range(S))
+    seen_c = sum(i % win + 1 for i in range(S))
+    io = T * H * (d + dv) * 2 + T * G * (d + dv) * 2
+    row("window_attention prefill (window %d, scores capped)" % win,
+        "window_attention prefill",
+        lambda: sk.window_attention(q, cache.pools[0], batch, G, d, dv,
+                                    d ** -0.5, win, 0, None, 0, 30.0),
+        io, 2.0 * B * H * seen_w * (d + dv), iters=2)
+    row("window_attention prefill (chunks of %d)" % win,
+        "window_attention prefill",
+        lambda: sk.window_attention(q, cache.pools[0], batch, G, d, dv,
+                                    d ** -0.5, 0, 0, None, win, 0.0),
+        io, 2.0 * B * H * seen_c * (d + dv), iters=2)
+    seen_l = sum(min(i + 1, win) + min(4, max(0, i + 1 - win))
+                 for i in range(S))
+    row("window_attention prefill (lolulorn: window %d + 4 kept)" % win, "",
+        lambda: sk.window_attention(q, cache.pools[0], batch, G, d, dv,
+                                    d ** -0.5, win, 4),
+        io, 2.0 * B * H * seen_l * (d + dv), iters=2)
+    cache.end_step()
+    # ---- decode attention at B and at 64 requests
+    for NB in (B, 64):
+        big = PagedStateCache([G * (d + dv)], {}, NB, NB * (S + 64), dtype=bf,
+                              device=dev)
+        big.pools[0].normal_()
+        for i in range(NB):
+            big.lens[i] = S - 1          # the last token of a full chunk
+        bt = big.begin_ragged(list(range(NB)), [1] * NB)
+        qd = (torch.randn(NB, H, d, device=dev) * 0.1).to(bf)
+        vis = min(S, win)
+        nbytes = NB * vis * G * (d + dv) * 2
+        row("window_attention decode (window, capped), %d requests" % NB,
+            "window_attention decode",
+            lambda: sk.window_attention(qd, big.pools[0], bt, G, d, dv,
+                                        d ** -0.5, win, 0, None, 0, 30.0),
+            nbytes)
+        row("window_attention decode (chunk), %d requests" % NB,
+            "window_attention decode",
+            lambda: sk.window_attention(qd, big.pools[0], bt, G, d, dv,
+                                        d ** -0.5, 0, 0, None, win, 0.0),
+            nbytes)
+        row("window_attention decode (lolulorn), %d requests" % NB, "",
+            lambda: sk.window_attention(qd, big.pools[0], bt, G, d, dv,
+                                        d ** -0.5, win, 4),
+            NB * min(S, win + 4) * G * (d + dv) * 2)
+        big.end_step()
+        del big
+    # ---- state-space prologue / epilogue against the delta rule's
+    MH, P, N, MG = 2 * W // 64, 64, 128, 8
+    inner, gn = MH * P, MG * N
+    C = inner + 2 * gn
+    rc = PagedStateCache([], {"conv": (3, C)}, B, B * (S + 64), dtype=bf,
+                         device=dev)
+    bt = rc.begin_ragged(list(range(B)), [S] * B)
+    pj = torch.randn(T, inner + C + MH, device=dev).to(bf)
+    cw = torch.randn(C, 4, device=dev).to(bf)
+    cb = torch.zeros(C, device=dev)
+    al, db = torch.zeros(MH, device=dev), torch.zeros(MH, device=dev)
+    row("ssd_prep (conv+bias+silu, dt, decay; fp32 out)", "delta_prep",
+        lambda: sk.ssd_prep(pj, bt, cw, cb, rc.states["conv"], al, db, MH, MG,
+                            N, P), T * (C * 2 + inner * 8 + gn * 8))
+    rc.end_step()
+    RH, RG, rd, rv = max(1, H // 2), max(1, H // 4), 128, 256
+    C2 = 2 * RG * rd + RH * rv
+    rc = PagedStateCache([], {"conv": (3, C2)}, B, B * (S + 64), dtype=bf,
+                         device=dev)
+    bt = rc.begin_ragged(list(range(B)), [S] * B)
+    pj2 = torch.randn(T, C2 + RH * rv + 2 * RH, device=dev).to(bf)
+    cw2 = torch.randn(C2, 4, device=dev).to(bf)
+    al2, db2 = torch.zeros(RH, device=dev), torch.zeros(RH, device=dev)
+    row("delta_prep (lolulorn)", "",
+        lambda: sk.delta_prep(pj2, bt, cw2, rc.states["conv"], al2, db2, RG,
+                              RH, rd, rv), T * C2 * 6)
+    rc.end_step()
+    o32 = torch.randn(T, MH, P, device=dev)
+    xx = torch.randn(T, MH, P, device=dev)
+    gate = torch.randn(T, inner, device=dev).to(bf)
+    skip = torch.ones(MH, device=dev)
+    gw = torch.ones(inner, device=dev)
+    row("gate_group_norm (fp32 o and x in, bf16 gate and out)",
+        "head_norm_gate",
+        lambda: sk.gate_group_norm(o32, xx, skip, gate, gw, 8, 1e-6, bf),
+        T * inner * 12)
+    o2 = torch.randn(T, RH, rv, device=dev)
+    gate2 = torch.randn(T, RH * rv, device=dev).to(bf)
+    nw = torch.ones(rv, device=dev)
+    row("head_norm_gate (lolulorn)", "",
+        lambda: sk.head_norm_gate(o2, nw, gate2, 1e-6, bf), T * RH * rv * 8)
+    del o32, xx, gate, o2, gate2, pj, pj2
+    # ---- the scans
+    ch, SN = W, 16
+    for NB, cnt in ((B, S), (B, 1), (64, 1)):
+        n = NB * cnt
+        rc = PagedStateCache([], {"rec": ((MH, N, P), torch.float32)}, NB,
+                             NB * (S + 64), dtype=bf, device=dev)
+        bt = rc.begin_ragged(list(range(NB)), [cnt] * NB)
+        qq = torch.randn(n, MG, N, device=dev) * 0.1
+        kk = torch.randn(n, MG, N, device=dev) * 0.1
+        vv = torch.randn(n, MH, P, device=dev)
+        dec = torch.rand(n, MH, device=dev) * 0.1 + 0.9
+        st = rc.states["rec"]
+        row("linear_scan mamba2 form, %d x %d tokens" % (NB, cnt),
+            "linear_scan",
+            lambda: sk.linear_scan(qq, kk, vv, dec, None, st, bt),
+            n * (2 * MG * N + 2 * MH * P) * 4 + 2 * NB * MH * N * P * 4)
+        rc.end_step()
+        del rc, qq, kk, vv
+        rc = PagedStateCache([], {"rec": ((ch, SN), torch.float32)}, NB,
+                             NB * (S + 64), dtype=bf, device=dev)
+        bt = rc.begin_ragged(list(range(NB)), [cnt] * NB)
+        xs = torch.randn(n, ch, device=dev).to(bf)
+        zs = torch.randn(n, ch, device=dev).to(bf)
+        bc = (torch.randn(n, 2 * SN, device=dev) * 0.1).to(bf)
+        dtp = torch.randn(n, ch, device=dev)
+        a_log = torch.zeros(ch, SN, device=dev)
+        zero = torch.zeros(ch, device=dev)
+        so = torch.empty(n, ch, device=dev, dtype=bf)
+        st2 = rc.states["rec"]
+        row("selective_scan, %d x %d tokens" % (NB, cnt), "linear_scan",
+            lambda: sk.selective_scan(xs, dtp, zero, a_log, bc[:, :SN],
+                                      bc[:, SN:], zero, zs, st2, bt, 1.0, so),
+            n * ch * 10 + n * 2 * SN * 2 + 2 * NB * ch * SN * 4)
+        rc.end_step()
+        del rc
+        rc = PagedStateCache([], {"rec": ((RH, rd, rv), torch.float32)}, NB,
+                             NB * (S + 64), dtype=bf, device=dev)
+        bt = rc.begin_ragged(list(range(NB)), [cnt] * NB)
+        qq = torch.randn(n, RG, rd, device=dev) * 0.1
+        kk = torch.nn.functional.normalize(
+            torch.randn(n, RG, rd, device=dev), dim=-1)
+        vv = torch.randn(n, RH, rv, device=dev)
+        dec = torch.rand(n, RH, device=dev) * 0.1 + 0.9
+        beta = torch.rand(n, RH, device=dev)
+        st3 = rc.states["rec"]
+        row("linear_scan delta (lolulorn), %d x %d tokens" % (NB, cnt), "",
+            lambda: sk.linear_scan(qq, kk, vv, dec, beta, st3, bt),
+            n * (2 * RG * rd + 2 * RH * rv) * 4 + 2 * NB * RH * rd * rv * 4)
+        rc.end_step()
+        del rc, qq, kk, vv
+    # ---- convolution of the selective scan's input, activations
+    rc = PagedStateCache([], {"conv": (3, ch)}, B, B * (S + 64), dtype=bf,
+                         device=dev)
+    bt = rc.begin_ragged(list(range(B)), [S] * B)
+    pin = torch.randn(T, 2 * ch + 64, device=dev).to(bf)
+    cw3 = torch.randn(ch, 4, device=dev).to(bf)
+    cb3 = torch.zeros(ch, device=dev)
+    row("conv_silu (bias, bf16 in and out, 4 taps)", "delta_prep",
+        lambda: sk.conv_silu_ragged(pin[:, 64:64 + ch], cw3,
+                                    rc.states["conv"], bt, cb3, bf),
+        T * ch * 4)
+    rc.end_step()
+    sd = torch.randn(T, 2 * W + F, device=dev).to(bf)
+    row("act_rows gelu_erf (column slice)", "glu",
+        lambda: sk.act_rows(sd[:, 2 * W:], 0), T * F * 4)
+    gu = torch.randn(T, 2 * F, device=dev).to(bf)
+    row("glu gelu_tanh (lolulorn)", "", lambda: sk.glu(gu, 1), T * F * 6)
+    return out
+
+
+def run_savovik(sizes=("s", "m", "l"), kernels=True):
+    dev = torch.device("cuda", torch.cuda.current_device())
+    report = {}
+    for name in sizes:
+        z = dict(SIZES[name])
+        z["layers"] = 4
+        rec = {"size": {k: z[k] for k in z},
+               "savovik": _ragged_throughput(savovik_config(z), z, dev),
+               "lolulorn": _ragged_throughput(lolulorn_config(z), z, dev),
+               "llama": _llama_throughput(z, dev)}
+        if kernels:
+            rows = _savovik_kernel_rows(z, dev)
+            rec["kernels"] = rows
+            like = {}
+            for r in rows:           # a sibling row follows the rows it is like
+                if not r["like"]:
+                    for q in rows:
+                        if q["like"] and q["like"] in r["kernel"] \
+                                and _same_case(q["kernel"], r["kernel"]):
+                            like[q["kernel"]] = q["distance"] / r["distance"]
+            rec["distance_over_sibling"] = like
+        report[name] = rec
+        torch.cuda.empty_cache()
+    return report
+
+
+def _same_case(a, b):
+    """Rows of one case carry the same '<n> requests' / '<n> x <m> tokens'."""
+    import re
+    pat = r"(\d+ requests|\d+ x \d+ tokens)"
+    return re.findall(pat, a) == re.findall(pat, b)
+
 def run(sizes=("s", "m", "l"), kernels=True):
     dev = torch.device("cuda", torch.cuda.current_device())
     report = {}
@@ -510,6 +805,24 @@ def run(sizes=("s", "m", "l"), kernels=True):
 
 def main(sizes="s,m,l", out=None, model="fizesun"):
     names = tuple(sizes.split(","))
+    if model == "savovik":
+        rep = run_savovik(names)
+        if out:
+            with open(out, "w") as f:
+                json.dump(rep, f, indent=1)
+        best = rep[names[-1]]
+        print(json.dumps({
+            "metric": "savovik_serving_tokens_per_s", "unit": "tokens/s",
+            "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+            "value": best["savovik"]["prefill_tok_s"],
+            "higher_is_better": True,
+            "sizes": {k: {"savovik": v["savovik"], "lolulorn": v["lolulorn"],
+                          "llama": v["llama"],
+                          "worst_distance_over_sibling": max(
+                              v.get("distance_over_sibling", {}).values(),
+                              default=None)}
+                      for k, v in rep.items()}}))
+        return rep
     rep = run(names) if model == "fizesun" else run_lolulorn(names)
     if out:
         with open(out, "w") as f:

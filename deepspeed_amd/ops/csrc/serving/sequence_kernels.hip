@@ -1305,16 +1305,270 @@ __global__ __launch_bounds__(NT) void gate_group_norm_k(
   }
 }
 
+// The same with eight columns per thread and the part kept in registers
+// between the two passes (part length a multiple of 8, at most 8 * NT * GGN).
+constexpr int GGN = 4;
+template <typename T>
+__global__ __launch_bounds__(NT) void gate_group_norm_vec_k(
+    const float* __restrict__ o, const float* __restrict__ x, const float* __restrict__ skip,
+    const T* __restrict__ gate, int ld_gate, const float* __restrict__ w, T* __restrict__ out,
+    int n, int vdim, int parts, float eps) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x, part = blockIdx.y;
+  const int len = n / parts, c0 = part * len;
+  const float* orow = o + (int64_t)t * n;
+  const float* xrow = x + (int64_t)t * n;
+  const T* grow = gate + (int64_t)t * ld_gate;
+  float y[GGN][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < GGN; ++i) {
+    const int c = c0 + (threadIdx.x + i * NT) * 8;
+    if (c < c0 + len) {
+      float xv[8], gv[8];
+      load8(orow + c, y[i]);
+      load8(xrow + c, xv);
+      load8(grow + c, gv);
+      const float sk = skip[c / vdim];  // vdim is a multiple of 8: one head per group
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y[i][e] = (y[i][e] + sk * xv[e]) * siluf_(gv[e]);
+        ss += y[i][e] * y[i][e];
+      }
+    }
+  }
+  const float inv = rsqrtf(block_sum(ss, red) / (float)len + eps);
+#pragma unroll
+  for (int i = 0; i < GGN; ++i) {
+    const int c = c0 + (threadIdx.x + i * NT) * 8;
+    if (c < c0 + len) {
+      float wv[8];
+      load8(w + c, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[i][e] *= inv * wv[e];
+      store8(out + (int64_t)t * n + c, y[i]);
+    }
+  }
+}
+
+// Eight neighbouring channels of the short convolution (+ bias) + SiLU at one
+// token: p points at the token's row of the convolved columns, sl at the
+// slot's tail. C, ld and the slot stride are multiples of 8.
+template <typename T, int TAPS>
+__device__ __forceinline__ void conv8_silu(const T* __restrict__ p, int ld,
+                                           const T* __restrict__ w,
+                                           const float* __restrict__ bias,
+                                           const T* __restrict__ sl, int C, int c, int j,
+                                           int pos, float (&acc)[8]) {
+  constexpr int TAIL = TAPS - 1;
+  float wv[8 * TAPS];  // channel-major: wv[e * TAPS + tap]
+#pragma unroll
+  for (int i = 0; i < TAPS; ++i) {
+    float tmp[8];
+    load8(w + (int64_t)c * TAPS + 8 * i, tmp);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) wv[8 * i + e] = tmp[e];
+  }
+  float x[8];
+  load8(p + c, x);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = wv[e * TAPS + TAIL] * x[e];
+#pragma unroll
+  for (int k = 1; k <= TAIL; ++k) {
+    if (pos - k >= 0) {  // block-uniform
+      if (k <= j)
+        load8(p - (int64_t)k * ld + c, x);
+      else
+        load8(sl + (int64_t)(TAIL + j - k) * C + c, x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += wv[e * TAPS + TAIL - k] * x[e];
+    }
+  }
+  if (bias) {
+    float bv[8];
+    load8(bias + c, bv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += bv[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
+}
+
+template <typename T, typename TO, int TAPS>
+__global__ __launch_bounds__(NT) void conv_silu_vec_k(
+    const T* __restrict__ x, int ld_x, const T* __restrict__ w, const float* __restrict__ bias,
+    const T* __restrict__ state, int64_t state_slot_stride, const int* __restrict__ cu,
+    const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
+    const int* __restrict__ tok_pos, TO* __restrict__ out, int C) {
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int j = t - cu[s];
+  const int pos = tok_pos[t];
+  const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  const T* p = x + (int64_t)t * ld_x;
+  for (int c = (blockIdx.y * NT + threadIdx.x) * 8; c < C; c += gridDim.y * NT * 8) {
+    float acc[8];
+    conv8_silu<T, TAPS>(p, ld_x, w, bias, sl, C, c, j, pos, acc);
+    store8(out + (int64_t)t * C + c, acc);
+  }
+}
+
+template <typename T, int TAPS>
+__global__ __launch_bounds__(NT) void ssd_prep_vec_k(
+    const T* __restrict__ proj, int ld_proj, const T* __restrict__ w,
+    const float* __restrict__ bias, const T* __restrict__ state, int64_t state_slot_stride,
+    const int* __restrict__ cu, const int* __restrict__ seq_slot,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    float* __restrict__ x_out, float* __restrict__ v_out, float* __restrict__ b_out,
+    float* __restrict__ c_out, float* __restrict__ decay, int H, int P, int G, int N) {
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int j = t - cu[s];
+  const int pos = tok_pos[t];
+  const int inner = H * P, gn = G * N;
+  const int C = inner + 2 * gn;
+  const T* sl = state + (int64_t)seq_slot[s] * state_slot_stride;
+  const T* p = proj + (int64_t)t * ld_proj + inner;  // the convolved columns
+  if (blockIdx.y == 0)
+    for (int h = threadIdx.x; h < H; h += NT)
+      decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * softplusf_(ld(p + C + h) + dt_bias[h]));
+  for (int c = (blockIdx.y * NT + threadIdx.x) * 8; c < C; c += gridDim.y * NT * 8) {
+    float y[8];
+    conv8_silu<T, TAPS>(p, ld_proj, w, bias, sl, C, c, j, pos, y);
+    if (c < inner) {
+      const int h = c / P;  // P is a multiple of 8: one head per group
+      const float dt = softplusf_(ld(p + C + h) + dt_bias[h]);
+      store8(x_out + (int64_t)t * inner + c, y);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] *= dt;
+      store8(v_out + (int64_t)t * inner + c, y);
+    } else if (c < inner + gn) {
+      store8(b_out + (int64_t)t * gn + c - inner, y);
+    } else {
+      store8(c_out + (int64_t)t * gn + c - inner - gn, y);
+    }
+  }
+}
+
+// The per-head prologue with eight values per lane: a head is shared by LG
+// lanes (a power of two, 8 * LG >= dim and vdim); all sizes multiples of 8.
+template <typename T, bool HALF, int LG>
+__global__ __launch_bounds__(NT) void attn_prep_heads_vec_k(
+    const T* __restrict__ proj, int ld_proj, const float* __restrict__ wq,
+    const float* __restrict__ wk, const int* __restrict__ tok_pos,
+    const int* __restrict__ tok_row, const float* __restrict__ cosT,
+    const float* __restrict__ sinT, T* __restrict__ pool, T* __restrict__ q_out, int H, int G,
+    int dim, int vdim, int rot_dims, int own_kv, int norm, float eps, float v_eps) {
+  const int t = blockIdx.x;
+  const int l = threadIdx.x % LG, grp = threadIdx.x / LG;
+  const T* p = proj + (int64_t)t * ld_proj;
+  const int nq = H * dim, nk = G * dim, nv = G * vdim;
+  const int half = rot_dims >> 1;
+  const float* cs = cosT + (int64_t)tok_pos[t] * half;
+  const float* sn = sinT + (int64_t)tok_pos[t] * half;
+  T* row = own_kv ? pool + (int64_t)tok_row[t] * (nk + nv) : nullptr;
+  const int jobs = own_kv ? H + 2 * G : H;
+  const int c0 = l * 8;
+  // every lane of a wave walks the same number of rounds: the group sums
+  // below use whole-wave shuffles
+  for (int j0 = 0; j0 < jobs; j0 += NT / LG) {
+    const int job = j0 + grp;
+    const bool have = job < jobs;
+    const bool is_v = have && job >= H + G;
+    const bool is_q = have && job < H;
+    const int n = is_v ? vdim : dim;
+    const T* in = p;
+    T* out = q_out;
+    if (is_q) {
+      in = p + job * dim;
+      out = q_out + (int64_t)t * nq + job * dim;
+    } else if (have && !is_v) {
+      in = p + nq + (job - H) * dim;
+      out = row + (job - H) * dim;
+    } else if (is_v) {
+      in = p + nq + nk + (job - H - G) * vdim;
+      out = row + nk + (job - H - G) * vdim;
+    }
+    const bool act = have && c0 < n;
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = 0.f;
+    if (act) load8(in + c0, x);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+    for (int o = 1; o < LG; o <<= 1) ss += __shfl_xor(ss, o, 64);
+    if (!act) continue;
+    if (is_v) {
+      if (v_eps >= 0.f) {
+        const float inv = rsqrtf(ss / (float)vdim + v_eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= inv;
+      }
+      store8(out + c0, x);
+      continue;
+    }
+    const float* w = is_q ? wq : wk;
+    const float inv = norm == 2 ? rsqrtf(ss / (float)dim + eps) : 1.f;
+    if (norm == 2) {
+      float wv[8];
+      load8(w + c0, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] *= inv * wv[e];
+    }
+    if (c0 < rot_dims) {
+      if (HALF) {  // the partner group sits half the rotated width away
+        const bool second = c0 >= half;
+        const int pc = second ? c0 - half : c0 + half;
+        const int f0 = second ? c0 - half : c0;
+        float o[8];
+        load8(in + pc, o);
+        if (norm == 2) {
+          float wv[8];
+          load8(w + pc, wv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] *= inv * wv[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float co = cs[f0 + e], si = sn[f0 + e];
+          x[e] = second ? x[e] * co + o[e] * si : x[e] * co - o[e] * si;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          if (c0 + e < rot_dims) {
+            const float co = cs[(c0 + e) >> 1], si = sn[(c0 + e) >> 1];
+            const float a = x[e], b = x[e + 1];
+            x[e] = a * co - b * si;
+            x[e + 1] = b * co + a * si;
+          }
+        }
+      }
+    }
+    store8(out + c0, x);
+  }
+}
+
 // --------------------------------------------------------- selective scan
-// One state vector S[c, 0..N) per channel, float. SR neighbouring lanes share
-// a channel, each holding NS consecutive states in registers (N <= NS * SR); a
-// block owns NT / SR channels of one sequence and walks its tokens in order:
+// One state vector S[c, 0..N) per channel, float. The 16 lanes of a DPP row
+// share a channel, each holding NS consecutive states in registers
+// (N <= 16 * NS); a block owns NT / 16 channels of one sequence and walks its
+// tokens in order:
 //   dt = softplus(dt_pre + dt_bias); S[n] = exp(dt * A[n]) * S[n] + dt * x * B[n];
 //   y = sum_n S[n] * C[n] + D * x; out = y * silu(z) * out_scale.
-// The sum runs lane-local in a fixed order, then over the SR lanes in a fixed
-// tree, so a result does not depend on where a sequence was cut. The next
-// token's operands are loaded while the current one is computed.
-template <typename T, int NS, int SR>
+// The operands of SCT tokens at a time are staged through LDS, double-buffered
+// (the next chunk's global loads are in flight while this chunk is computed);
+// the staging thread also evaluates softplus and silu, once per channel and
+// token. The sum runs lane-local in a fixed order, then over the 16 lanes in
+// a fixed DPP tree, so a result does not depend on where a sequence was cut.
+// A is kept times log2(e): the decay is one multiply and one exp2.
+constexpr int SCH = NT / 16;  // channels per block
+constexpr int SCT = 16;       // tokens per staged chunk
+
+template <typename T, int NS>
 __global__ __launch_bounds__(NT) void selective_scan_k(
     const T* __restrict__ x, int ld_x, const float* __restrict__ dt_pre,
     const float* __restrict__ dt_bias, const float* __restrict__ a_log,
@@ -1322,9 +1576,18 @@ __global__ __launch_bounds__(NT) void selective_scan_k(
     const float* __restrict__ skip, const T* __restrict__ z, int ld_z,
     float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ seq_slot,
     T* __restrict__ out, int ld_out, int ch, int N, float out_scale) {
+  constexpr int NP = 16 * NS;  // padded state size
+  __shared__ float sDt[2][SCT][SCH];
+  __shared__ float sX[2][SCT][SCH];
+  __shared__ float sG[2][SCT][SCH];
+  __shared__ __attribute__((aligned(16))) float sB[2][SCT][NP];
+  __shared__ __attribute__((aligned(16))) float sC[2][SCT][NP];
+  __shared__ float sO[SCT][SCH];
   const int s = blockIdx.x;
-  const int r = threadIdx.x % SR;
-  const int c_raw = blockIdx.y * (NT / SR) + threadIdx.x / SR;
+  const int r = threadIdx.x & 15;
+  const int cl = threadIdx.x >> 4;
+  const int c0 = blockIdx.y * SCH;
+  const int c_raw = c0 + cl;
   const bool live = c_raw < ch;
   const int c = live ? c_raw : ch - 1;  // idle lanes shadow the last channel
   const int n0 = r * NS;
@@ -1334,43 +1597,86 @@ __global__ __launch_bounds__(NT) void selective_scan_k(
   for (int i = 0; i < NS; ++i) {
     const bool in = n0 + i < N;
     S[i] = in ? Sg[n0 + i] : 0.f;
-    A[i] = in ? -expf(a_log[(int64_t)c * N + n0 + i]) : 0.f;
+    A[i] = in ? -expf(a_log[(int64_t)c * N + n0 + i]) * 1.4426950408889634f : 0.f;
   }
-  const float bias = dt_bias[c], dsk = skip[c];
+  const float dsk = skip[c];
   const int t0 = cu[s], n = cu[s + 1] - t0;
-  float nb[NS], nc[NS], ndt = 0.f, nx = 0.f, nz = 0.f;
-  auto fetch = [&](int t) {
-    ndt = dt_pre[(int64_t)t * ch + c];
-    nx = ld(x + (int64_t)t * ld_x + c);
-    nz = ld(z + (int64_t)t * ld_z + c);
+  const int nchunks = (n + SCT - 1) / SCT;
+
+  // staging: element f of a chunk's [SCT][SCH] block is (token f / SCH,
+  // channel f % SCH); of its [SCT][NP] block (token f / NP, state f % NP)
+  constexpr int EPT = SCT * SCH / NT;              // = 1
+  constexpr int BPT = (SCT * NP + NT - 1) / NT;    // = NS
+  float pdt[EPT], px[EPT], pz[EPT], pb[BPT], pc[BPT];
+  auto fetch = [&](int k) {
+    const int nt = min(SCT, n - k * SCT);
+    const int tc = t0 + k * SCT;
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const bool in = n0 + i < N;
-      nb[i] = in ? ld(Bm + (int64_t)t * ld_bc + n0 + i) : 0.f;
-      nc[i] = in ? ld(Cm + (int64_t)t * ld_bc + n0 + i) : 0.f;
+    for (int i = 0; i < EPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / SCH, e = c0 + f % SCH;
+      const bool in = tk < nt && e < ch;
+      pdt[i] = in ? dt_pre[(int64_t)(tc + tk) * ch + e] + dt_bias[e] : 0.f;
+      px[i] = in ? ld(x + (int64_t)(tc + tk) * ld_x + e) : 0.f;
+      pz[i] = in ? ld(z + (int64_t)(tc + tk) * ld_z + e) : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < BPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / NP, e = f % NP;
+      const bool in = tk < nt && e < N;
+      pb[i] = in ? ld(Bm + (int64_t)(tc + tk) * ld_bc + e) : 0.f;
+      pc[i] = in ? ld(Cm + (int64_t)(tc + tk) * ld_bc + e) : 0.f;
     }
   };
-  if (n > 0) fetch(t0);
-  for (int k = 0; k < n; ++k) {
-    const float dt = softplusf_(ndt + bias), xv = nx, zv = nz;
-    float b[NS], cc[NS];
+  auto stash = [&](int b) {
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      b[i] = nb[i];
-      cc[i] = nc[i];
-    }
-    if (k + 1 < n) fetch(t0 + k + 1);
-    const float dx = dt * xv;
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      S[i] = expf(dt * A[i]) * S[i] + dx * b[i];
-      acc += S[i] * cc[i];
+    for (int i = 0; i < EPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / SCH, e = f % SCH;
+      sDt[b][tk][e] = softplusf_(pdt[i]);
+      sX[b][tk][e] = px[i];
+      sG[b][tk][e] = siluf_(pz[i]) * out_scale;
     }
 #pragma unroll
-    for (int o = 1; o < SR; o <<= 1) acc += __shfl_xor(acc, o, 64);
-    if (live && r == 0)
-      st(out + (int64_t)(t0 + k) * ld_out + c, (acc + dsk * xv) * siluf_(zv) * out_scale);
+    for (int i = 0; i < BPT; ++i) {
+      const int f = threadIdx.x + i * NT;
+      const int tk = f / NP, e = f % NP;
+      if (tk < SCT) {
+        sB[b][tk][e] = pb[i];
+        sC[b][tk][e] = pc[i];
+      }
+    }
+  };
+  if (nchunks > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int k = 0; k < nchunks; ++k) {
+    const int b = k & 1;
+    if (k + 1 < nchunks) fetch(k + 1);
+    const int nt = min(SCT, n - k * SCT);
+    for (int tk = 0; tk < nt; ++tk) {
+      const float dt = sDt[b][tk][cl], xv = sX[b][tk][cl];
+      const float dx = dt * xv;
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        S[i] = __builtin_amdgcn_exp2f(dt * A[i]) * S[i] + dx * sB[b][tk][n0 + i];
+        acc += S[i] * sC[b][tk][n0 + i];
+      }
+      acc = group_sum(acc);
+      if (r == 0) sO[tk][cl] = (acc + dsk * xv) * sG[b][tk][cl];
+    }
+    __syncthreads();  // sO complete; every lane is done with buffer b
+    {  // the chunk's results, channel-contiguous
+      const int f = threadIdx.x;
+      const int tk = f / SCH, e = c0 + f % SCH;
+      if (tk < nt && e < ch) st(out + (int64_t)(t0 + k * SCT + tk) * ld_out + e, sO[tk][f % SCH]);
+    }
+    if (k + 1 < nchunks) stash(b ^ 1);
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -1555,6 +1861,30 @@ int dsv_attn_prep_heads(const void* proj, int ld_proj, const float* wq, const fl
   if ((norm != 0 && norm != 2) || (norm == 2 && (!wq || (own_kv && !wk)))) return -2;
   if (rot_dims > 0 && (!cosT || !sinT)) return -3;
   if (Ttok <= 0) return 0;
+  const int big = dim > vdim ? dim : vdim;
+  // vector form: whole groups of 8 everywhere; with the half pairing a group's
+  // partner is a whole group too
+  const bool vec = dim % 8 == 0 && vdim % 8 == 0 && ld_proj % 8 == 0 && big <= 512 &&
+                   (half ? rot_dims % 16 == 0 : true) && (uintptr_t)proj % 16 == 0;
+#define PREPH(HALF, LG)                                                                        \
+  BY_DTYPE(dt, (attn_prep_heads_vec_k<T, HALF, LG><<<Ttok, NT, 0, s>>>(                         \
+                   (const T*)proj, ld_proj, wq, wk, tok_pos, tok_row, cosT, sinT, (T*)pool,    \
+                   (T*)q_out, H, G, dim, vdim, rot_dims, own_kv, norm, eps, v_eps)))
+#define PREPH_BY_LG(HALF)                        \
+  do {                                           \
+    if (big <= 32) PREPH(HALF, 4);               \
+    else if (big <= 64) PREPH(HALF, 8);          \
+    else if (big <= 128) PREPH(HALF, 16);        \
+    else if (big <= 256) PREPH(HALF, 32);        \
+    else PREPH(HALF, 64);                        \
+  } while (0)
+  if (vec) {
+    if (half) PREPH_BY_LG(true);
+    else PREPH_BY_LG(false);
+    return (int)hipGetLastError();
+  }
+#undef PREPH_BY_LG
+#undef PREPH
   if (half)
     BY_DTYPE(dt, (attn_prep_heads_k<T, true><<<Ttok, NT, 0, s>>>(
                      (const T*)proj, ld_proj, wq, wk, tok_pos, tok_row, cosT, sinT, (T*)pool,
@@ -1573,7 +1903,25 @@ int dsv_conv_silu(const void* x, int ld_x, const void* w, const float* bias, voi
                   int dt, int out_dt, int Ttok, int nseq, int C, int taps, hipStream_t s) {
   if (taps < 1 || taps > MAXTAPS_SEQ || ld_x < C) return -1;
   if (Ttok <= 0) return 0;
-  if (out_dt == 0)
+  const bool vec = C % 8 == 0 && ld_x % 8 == 0 && state_slot_stride % 8 == 0 &&
+                   (uintptr_t)x % 16 == 0 && taps >= 2 && taps <= 4;
+  const dim3 grid(Ttok, Ttok < 512 ? (C / 8 + NT - 1) / NT : 1);
+#define CONVV(TAPS)                                                                             \
+  do {                                                                                          \
+    if (out_dt == 0)                                                                            \
+      BY_DTYPE(dt, (conv_silu_vec_k<T, float, TAPS><<<grid, NT, 0, s>>>(                         \
+                       (const T*)x, ld_x, (const T*)w, bias, (const T*)state,                   \
+                       state_slot_stride, cu, seq_slot, tok_seq, tok_pos, (float*)out, C)));    \
+    else                                                                                        \
+      BY_DTYPE(dt, (conv_silu_vec_k<T, T, TAPS><<<grid, NT, 0, s>>>(                             \
+                       (const T*)x, ld_x, (const T*)w, bias, (const T*)state,                   \
+                       state_slot_stride, cu, seq_slot, tok_seq, tok_pos, (T*)out, C)));        \
+  } while (0)
+  if (vec && taps == 4) CONVV(4);
+  else if (vec && taps == 3) CONVV(3);
+  else if (vec && taps == 2) CONVV(2);
+  else if (out_dt == 0)
+#undef CONVV
     BY_DTYPE(dt, (conv_silu_k<T, float><<<Ttok, NT, 0, s>>>(
                      (const T*)x, ld_x, (const T*)w, bias, (const T*)state, state_slot_stride,
                      cu, seq_slot, tok_seq, tok_pos, (float*)out, C, taps)));
@@ -1598,6 +1946,20 @@ int dsv_ssd_prep(const void* proj, int ld_proj, const void* w, const float* bias
   if (ld_proj < 2 * H * P + 2 * G * N + H) return -2;
   if (Ttok <= 0) return 0;
   const int inner = H * P, C = inner + 2 * G * N;
+  const bool vec = P % 8 == 0 && (G * N) % 8 == 0 && ld_proj % 8 == 0 &&
+                   state_slot_stride % 8 == 0 && (uintptr_t)proj % 16 == 0 && taps >= 2 &&
+                   taps <= 4;
+  const dim3 grid(Ttok, Ttok < 512 ? (C / 8 + NT - 1) / NT : 1);
+#define SSDV(TAPS)                                                                             \
+  BY_DTYPE(dt, (ssd_prep_vec_k<T, TAPS><<<grid, NT, 0, s>>>(                                    \
+                   (const T*)proj, ld_proj, (const T*)w, bias, (const T*)state,                \
+                   state_slot_stride, cu, seq_slot, tok_seq, tok_pos, a_log, dt_bias, x_out,   \
+                   v_out, b_out, c_out, decay, H, P, G, N)))
+  if (vec && taps == 4) SSDV(4);
+  else if (vec && taps == 3) SSDV(3);
+  else if (vec && taps == 2) SSDV(2);
+  else
+#undef SSDV
   BY_DTYPE(dt, (ssd_prep_k<T><<<Ttok, NT, H * sizeof(float), s>>>(
                    (const T*)proj, ld_proj, (const T*)w, bias, (const T*)state,
                    state_slot_stride, cu, seq_slot, tok_seq, tok_pos, a_log, dt_bias, x_out,
@@ -1615,8 +1977,14 @@ int dsv_gate_group_norm(const float* o, const float* x, const float* skip, const
   const int n = H * vdim;
   if (parts < 1 || n % parts || ld_gate < n) return -1;
   if (Ttok <= 0) return 0;
-  BY_DTYPE(dt, (gate_group_norm_k<T><<<dim3(Ttok, parts), NT, 0, s>>>(
-                   o, x, skip, (const T*)gate, ld_gate, w, (T*)out, n, vdim, parts, eps)));
+  const int len = n / parts;
+  if (len % 8 == 0 && vdim % 8 == 0 && ld_gate % 8 == 0 && len <= 8 * NT * GGN &&
+      (uintptr_t)gate % 16 == 0)
+    BY_DTYPE(dt, (gate_group_norm_vec_k<T><<<dim3(Ttok, parts), NT, 0, s>>>(
+                     o, x, skip, (const T*)gate, ld_gate, w, (T*)out, n, vdim, parts, eps)));
+  else
+    BY_DTYPE(dt, (gate_group_norm_k<T><<<dim3(Ttok, parts), NT, 0, s>>>(
+                     o, x, skip, (const T*)gate, ld_gate, w, (T*)out, n, vdim, parts, eps)));
   return (int)hipGetLastError();
 }
 
@@ -1631,19 +1999,19 @@ int dsv_selective_scan(const void* x, int ld_x, const float* dt_pre, const float
   if (N < 1 || N > dsv_selective_scan_max_state() || ch < 1) return -1;
   if (ld_x < ch || ld_z < ch || ld_out < ch || ld_bc < N) return -2;
   if (nseq <= 0) return 0;
-#define SSCAN(NS, SR)                                                                          \
+#define SSCAN(NS)                                                                              \
   do {                                                                                         \
-    dim3 grid(nseq, (ch + NT / SR - 1) / (NT / SR));                                           \
-    BY_DTYPE(dt, (selective_scan_k<T, NS, SR><<<grid, NT, 0, s>>>(                              \
+    dim3 grid(nseq, (ch + SCH - 1) / SCH);                                                     \
+    BY_DTYPE(dt, (selective_scan_k<T, NS><<<grid, NT, 0, s>>>(                                  \
                      (const T*)x, ld_x, dt_pre, dt_bias, a_log, (const T*)Bm, (const T*)Cm,    \
                      ld_bc, skip, (const T*)z, ld_z, state, cu, seq_slot, (T*)out, ld_out, ch, \
                      N, out_scale)));                                                          \
   } while (0)
-  if (N <= 16) SSCAN(4, 4);
-  else if (N <= 32) SSCAN(8, 4);
-  else if (N <= 64) SSCAN(16, 4);
-  else if (N <= 128) SSCAN(16, 8);
-  else SSCAN(16, 16);
+  if (N <= 16) SSCAN(1);
+  else if (N <= 32) SSCAN(2);
+  else if (N <= 64) SSCAN(4);
+  else if (N <= 128) SSCAN(8);
+  else SSCAN(16);
 #undef SSCAN
   return (int)hipGetLastError();
 }
