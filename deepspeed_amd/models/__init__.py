@@ -11,6 +11,7 @@ from .falcon import (FalconConfig, FalconForCausalLM, falcon_7b,
 from .mixtral import (MixtralConfig, MixtralForCausalLM, mixtral_8x7b,
                       mixtral_tiny, mixtral_mini)
 from .fizesun import FizesunConfig, FizesunForCausalLM, fizesun_tiny
+from .savovik import SavovikConfig, SavovikForCausalLM, savovik_tiny
 from .registry import (architectures, build_model, load_pretrained,
                        register_architecture)
 
@@ -24,6 +25,7 @@ __all__ = [
     "MixtralConfig", "MixtralForCausalLM",
     "mixtral_8x7b", "mixtral_tiny", "mixtral_mini",
     "FizesunConfig", "FizesunForCausalLM", "fizesun_tiny",
+    "SavovikConfig", "SavovikForCausalLM", "savovik_tiny",
     "architectures", "build_model", "load_pretrained",
     "register_architecture",
 ]
