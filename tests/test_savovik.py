@@ -556,6 +556,41 @@ def test_selective_scan_keeps_a_far_input_by_its_decay():
         assert float(got[2].abs().max()) == 0.0
 
 
+def test_matrix_state_keeps_a_far_input_by_its_decay():
+    """Scalar-decay recurrence through its prologue: one input at token 3,
+    silence afterwards, constant B, C and step size; 200 tokens later the
+    read-out is that input times the 200th power of the decay, whether the
+    tokens come at once or one by one."""
+    from deepspeed_amd.ops.linear_recurrence import linear_scan, ssd_prep
+    T, H, P, G, N = 204, 1, 2, 1, 2
+    proj = torch.zeros(T, 2 * H * P + 2 * G * N + H)
+    proj[3, 2:4] = torch.tensor([1.0, -2.0])          # x before SiLU
+    proj[:, 4:8] = 1.5                                 # B and C before SiLU
+    proj[:, 8] = 0.3
+    w, bias = torch.ones(H * P + 2 * G * N, 1), torch.zeros(H * P + 2 * G * N)
+    a_log, dt_bias = torch.tensor([-2.0]), torch.tensor([-0.1])
+    dt = math.log1p(math.exp(0.2))
+    a = math.exp(-math.exp(-2.0) * dt)
+    bc = float(O.silu(torch.tensor(1.5, dtype=torch.float64)))
+    x3 = O.silu(torch.tensor([1.0, -2.0], dtype=torch.float64))
+    want = N * bc * bc * dt * x3 * a ** 200
+    for cuts in ([T], [4] + [1] * 200):
+        cache = PagedStateCache([], {"conv": (0, H * P + 2 * G * N),
+                                     "rec": ((H, N, P), torch.float32)}, 1,
+                                256, block_size=8, device=DEV)
+
+        def step(b, lo, hi):
+            Cq, Bk, v, x, decay = ssd_prep(
+                proj[lo:hi].to(DEV), b, w.to(DEV), bias.to(DEV),
+                cache.states["conv"], a_log.to(DEV), dt_bias.to(DEV), H, G, N,
+                P)
+            return linear_scan(Cq, Bk, v, decay, None, cache.states["rec"],
+                               b).cpu().double().reshape(hi - lo, P)
+        got = in_steps(cache, 0, cuts, step)
+        close(got[203], want, 1e-4)
+        assert float(got[2].abs().max()) == 0.0
+
+
 def test_short_convolution_with_bias_tail_carried_and_zero_at_the_start():
     from deepspeed_amd.ops.causal_conv import conv_silu_ragged
     torch.manual_seed(0)
@@ -1026,3 +1061,92 @@ def test_attention_kernel_masks_against_eager(dtype, heads, kv, dim, vdim,
     tol = 1e-4 if dtype == torch.float32 else 2e-2
     assert (got - want).abs().max().item() < tol * max(1.0, want.abs().max()
                                                        .item())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,dim,vdim,dims,layout,norm,unit", [
+    (8, 2, 128, 128, 64, "half", None, True),
+    (8, 2, 128, 64, 64, "interleaved", "head", False),
+    (4, 4, 256, 256, 128, "half", "head", True),
+    (6, 3, 64, 32, 64, "interleaved", None, False),
+    (3, 1, 40, 24, 16, "half", "head", True),
+    (2, 2, 36, 20, 10, "half", "head", True),           # scalar form
+    (5, 5, 48, 48, 24, "half", None, True)])            # half not a multiple of 8
+def test_attention_prologue_sizes_against_eager(dtype, heads, kv, dim, vdim,
+                                                dims, layout, norm, unit,
+                                                monkeypatch):
+    from deepspeed_amd.ops import window_attention as wa
+    from deepspeed_amd.ops.rope import rope_tables
+    g = torch.Generator().manual_seed(dim + vdim)
+    held, counts = [5, 100], [40, 1]
+    T = sum(counts)
+    n = heads * dim + kv * (dim + vdim)
+    wide = (torch.randn(T, n + 16, generator=g) * 2).to(dtype).to(DEV)
+    proj = wide[:, 8:8 + n]                     # a column slice
+    wq = (1 + 0.2 * torch.randn(dim, generator=g)).to(DEV)
+    wk = (1 + 0.2 * torch.randn(dim, generator=g)).to(DEV)
+    outs = []
+    for eager in (False, True):
+        if eager:
+            monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+        cache, b = one_step_cache([kv * (dim + vdim)], {}, held, counts,
+                                  block=64, tokens=64 * 8)
+        cache.pools[0] = cache.pools[0].to(dtype)
+        cos, sin = rope_tables(dims, cache.max_seq, 1000.0, device=DEV,
+                               scaling=2.0)
+        q = wa.attn_prep(proj, b, cache.pools[0], wq, wk, 1e-5, heads, kv,
+                         dim, vdim, dims, cos, sin, True, norm, layout,
+                         1e-5 if unit else None)
+        outs.append((q.float().cpu(), cache.pools[0].float().cpu()))
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for got, want in zip(*outs):
+        assert (got - want).abs().max().item() < tol * max(
+            1.0, want.abs().max().item())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,vdim,state,groups,parts,taps", [
+    (8, 64, 128, 2, 4, 4), (4, 16, 24, 4, 1, 3), (6, 8, 20, 3, 2, 2),
+    (4, 32, 64, 1, 8, 5), (3, 5, 7, 3, 3, 4), (2, 64, 256, 2, 2, 1)])
+def test_state_space_prologue_and_epilogue_against_eager(
+        dtype, heads, vdim, state, groups, parts, taps, monkeypatch):
+    from deepspeed_amd.ops.linear_recurrence import gate_group_norm, ssd_prep
+    g = torch.Generator().manual_seed(heads * vdim + state)
+    counts = [37, 1, 2]
+    T = sum(counts)
+    inner, C = heads * vdim, heads * vdim + 2 * groups * state
+    proj = torch.randn(T, inner + C + heads, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(C, taps, generator=g) * 0.5).to(dtype).to(DEV)
+    bias = torch.randn(C, generator=g).to(DEV)
+    a_log, dt_bias = torch.randn(heads, generator=g).to(DEV), \
+        torch.randn(heads, generator=g).to(DEV)
+    skip, nw = torch.randn(heads, generator=g).to(DEV), \
+        torch.randn(inner, generator=g).to(DEV)
+    tail0 = torch.randn(3, max(taps - 1, 0), C, generator=g).to(dtype)
+    held = (9, 70, 1)
+    for slot, n in enumerate(held):             # nothing before position 0
+        tail0[slot, :max(0, taps - 1 - n)] = 0
+    outs = []
+    for eager in (False, True):
+        if eager:
+            monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+        cache = PagedStateCache([], {"conv": ((max(taps - 1, 0), C), dtype)},
+                                3, 512, block_size=64, device=DEV)
+        cache.states["conv"].copy_(tail0)
+        for slot, n in enumerate(held):
+            cache.lens[slot] = n
+        b = cache.begin_ragged([0, 1, 2], counts)
+        Cq, Bk, v, x, decay = ssd_prep(proj, b, w, bias, cache.states["conv"],
+                                       a_log, dt_bias, heads, groups, state,
+                                       vdim)
+        y = gate_group_norm(v.contiguous(), x, skip, proj[:, :inner], nw,
+                            parts, 1e-5, dtype)
+        outs.append([t.float().cpu() for t in
+                     (Cq, Bk, v, x, decay, y, cache.states["conv"])])
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for got, want in zip(*outs):
+        if want.numel():                        # one tap keeps no tail
+            assert (got - want).abs().max().item() < tol * max(
+                1.0, want.abs().max().item())
