@@ -966,6 +966,35 @@ def test_generate_command_line(tmp_path):
         assert line["generated"] == seq[len(prompt):]
 
 
+def test_http_server_generates_the_oracles_tokens():
+    """The FastAPI front end over the same scheduler: concurrent requests,
+    greedy tokens as the oracle's."""
+    from concurrent.futures import ThreadPoolExecutor
+    from fastapi.testclient import TestClient
+    from deepspeed_amd.inference.server import InferenceServer, build_app
+    s = Served(BASE, seed=21)
+    prompts = [toks(n, seed=90 + n) for n in (5, 9, 3)]
+    server = InferenceServer(s.model, max_slots=2).start()
+    try:
+        client = TestClient(build_app(server))
+
+        def call(p):
+            r = client.post("/generate", json={"token_ids": p,
+                                               "max_new_tokens": 4})
+            assert r.status_code == 200
+            return r.json()["generated"]
+
+        with ThreadPoolExecutor(3) as ex:
+            got = list(ex.map(call, prompts))
+    finally:
+        server.stop()
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        for _ in range(4):
+            seq.append(int(s.oracle(seq)[-1].argmax()))
+        assert g == seq[len(p):]
+
+
 # ------------------------------------------- HIP kernels against eager ops
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
