@@ -12,6 +12,7 @@ from .mixtral import (MixtralConfig, MixtralForCausalLM, mixtral_8x7b,
                       mixtral_tiny, mixtral_mini)
 from .fizesun import FizesunConfig, FizesunForCausalLM, fizesun_tiny
 from .savovik import SavovikConfig, SavovikForCausalLM, savovik_tiny
+from .numolorn import NumolornConfig, NumolornForCausalLM, numolorn_tiny
 from .registry import (architectures, build_model, load_pretrained,
                        register_architecture)
 
@@ -26,6 +27,7 @@ __all__ = [
     "mixtral_8x7b", "mixtral_tiny", "mixtral_mini",
     "FizesunConfig", "FizesunForCausalLM", "fizesun_tiny",
     "SavovikConfig", "SavovikForCausalLM", "savovik_tiny",
+    "NumolornConfig", "NumolornForCausalLM", "numolorn_tiny",
     "architectures", "build_model", "load_pretrained",
     "register_architecture",
 ]

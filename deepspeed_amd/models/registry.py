@@ -92,6 +92,7 @@ def _register_builtin():
     from .llama import LlamaConfig, LlamaForCausalLM
     from .lolulorn import build_from_config as build_lolulorn
     from .mixtral import MixtralConfig, MixtralForCausalLM
+    from .numolorn import build_from_config as build_numolorn
     from .savovik import build_from_config as build_savovik
     hf = {"num_hidden_layers": "num_layers",
           "num_attention_heads": "num_heads",
@@ -110,6 +111,7 @@ def _register_builtin():
             FizesunConfig.from_dict(cfg), dtype))
     register_architecture("Lolulorn", build_lolulorn, wants_tensors=True)
     register_architecture("Savovik", build_savovik)
+    register_architecture("Numolorn", build_numolorn, wants_tensors=True)
 
 
 _register_builtin()

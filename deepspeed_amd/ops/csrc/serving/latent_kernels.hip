@@ -13,60 +13,73 @@
 namespace {
 
 // ------------------------------------------------------ latent prologue
-// proj row = [ q (H x (dim+rot)) | latent (rank) | k_rot (rot) | gate (H) ].
+// Three row sources (each a column slice with a row stride of its own, so they
+// may be parts of one projection or come from different products):
+//   q    = [ H x (dim + rot) ]      kv = [ latent (rank) | k_rot (rot) ]
+//   gate = [ H ] logits, or null (no gate output)
+// HALF pairs coordinate i with i + rot_dims/2 among the first rot_dims of a
+// rotated part; otherwise neighbours (2i, 2i+1) form a pair.
 template <typename T>
 __global__ __launch_bounds__(NT) void latent_prep_k(
-    const T* __restrict__ proj, int ld_proj, const float* __restrict__ norm_w,
+    const T* __restrict__ q_src, int ld_q, const T* __restrict__ kv_src, int ld_kv,
+    const T* __restrict__ gate_src, int ld_g, const float* __restrict__ norm_w,
     const int* __restrict__ tok_pos, const int* __restrict__ tok_row,
     const float* __restrict__ cosT, const float* __restrict__ sinT,
     T* __restrict__ pool, T* __restrict__ q_nope, T* __restrict__ q_rot,
     float* __restrict__ gate, int Ttok, int H, int dim, int rot, int rank,
-    int rot_dims, float eps) {
+    int rot_dims, float eps, int half_layout) {
   __shared__ float red[NT / 64];
   const int t = blockIdx.x;
-  const T* p = proj + (int64_t)t * ld_proj;
-  const int nq = H * (dim + rot);
+  const T* pq = q_src + (int64_t)t * ld_q;
+  const T* pkv = kv_src + (int64_t)t * ld_kv;
   const int half = rot_dims >> 1;
-  const float* cs = cosT + (int64_t)tok_pos[t] * half;
-  const float* sn = sinT + (int64_t)tok_pos[t] * half;
+  const float* cs = rot_dims ? cosT + (int64_t)tok_pos[t] * half : nullptr;
+  const float* sn = rot_dims ? sinT + (int64_t)tok_pos[t] * half : nullptr;
   T* row = pool + (int64_t)tok_row[t] * (rank + rot);
   float ss = 0.f;
   for (int c = threadIdx.x; c < rank; c += NT) {
-    float v = ld(p + nq + c);
+    float v = ld(pkv + c);
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float k = rsqrtf(ss / (float)rank + eps);
   for (int c = threadIdx.x; c < rank; c += NT)
-    st(row + c, ld(p + nq + c) * k * norm_w[c]);
-  // shared rotated key part
-  for (int c = threadIdx.x; c < rot; c += NT) {
-    float v = ld(p + nq + rank + c);
+    st(row + c, ld(pkv + c) * k * norm_w[c]);
+  // one coordinate of a rotated part: its partner, its pair and its side
+  auto turn = [&](const T* src, int c) -> float {
+    float v = ld(src + c);
     if (c < rot_dims) {
-      const float o = ld(p + nq + rank + (c ^ 1));
-      const float co = cs[c >> 1], si = sn[c >> 1];
-      v = (c & 1) ? v * co + o * si : v * co - o * si;
+      int partner, pair;
+      bool second;
+      if (half_layout) {
+        second = c >= half;
+        partner = second ? c - half : c + half;
+        pair = second ? c - half : c;
+      } else {
+        second = c & 1;
+        partner = c ^ 1;
+        pair = c >> 1;
+      }
+      const float o = ld(src + partner);
+      const float co = cs[pair], si = sn[pair];
+      v = second ? v * co + o * si : v * co - o * si;
     }
-    st(row + rank + c, v);
-  }
+    return v;
+  };
+  // shared rotated key part
+  for (int c = threadIdx.x; c < rot; c += NT) st(row + rank + c, turn(pkv + rank, c));
   // queries: rotated part [T, H, rot]; unrotated part regrouped [H, T, dim]
   for (int i = threadIdx.x; i < H * rot; i += NT) {
     const int h = i / rot, c = i - h * rot;
-    const T* q = p + h * (dim + rot) + dim;
-    float v = ld(q + c);
-    if (c < rot_dims) {
-      const float o = ld(q + (c ^ 1));
-      const float co = cs[c >> 1], si = sn[c >> 1];
-      v = (c & 1) ? v * co + o * si : v * co - o * si;
-    }
-    st(q_rot + ((int64_t)t * H + h) * rot + c, v);
+    st(q_rot + ((int64_t)t * H + h) * rot + c, turn(pq + h * (dim + rot) + dim, c));
   }
   for (int i = threadIdx.x; i < H * dim; i += NT) {
     const int h = i / dim, c = i - h * dim;
-    q_nope[((int64_t)h * Ttok + t) * dim + c] = p[h * (dim + rot) + c];
+    q_nope[((int64_t)h * Ttok + t) * dim + c] = pq[h * (dim + rot) + c];
   }
-  for (int h = threadIdx.x; h < H; h += NT)
-    gate[(int64_t)t * H + h] = 1.f / (1.f + expf(-ld(p + nq + rank + rot + h)));
+  if (gate_src)
+    for (int h = threadIdx.x; h < H; h += NT)
+      gate[(int64_t)t * H + h] = 1.f / (1.f + expf(-ld(gate_src + (int64_t)t * ld_g + h)));
 }
 
 // ------------------------------------------------------ latent attention
@@ -87,7 +100,8 @@ __global__ __launch_bounds__(NT) void latent_attn_k(
     const int* __restrict__ table, int maxb, int bs,
     T* __restrict__ out,          // [H, Ttok, rank]
     float* __restrict__ part,     // [Ttok, nsplit, H, rank + 2] when nsplit > 1
-    int Ttok, int H, int rank, int rot, int KC, int nsplit, float scale) {
+    int Ttok, int H, int rank, int rot, int KC, int nsplit, float scale, int window,
+    const float* __restrict__ sink) {
   extern __shared__ float smem[];
   const int D = rank + rot;
   const int DS = D | 1;
@@ -100,7 +114,9 @@ __global__ __launch_bounds__(NT) void latent_attn_k(
   const int t = blockIdx.x, split = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const int s = tok_seq[t];
-  const int nkeys = tok_pos[t] + 1;
+  // visible keys klo .. tok_pos[t]; chunks count from klo
+  const int klo = window > 0 ? max(0, tok_pos[t] + 1 - window) : 0;
+  const int nkeys = tok_pos[t] + 1 - klo;
   const int* tab = table + (int64_t)s * maxb;
   // key range of this split, in whole chunks
   const int nchunk = (nkeys + KC - 1) / KC;
@@ -130,7 +146,7 @@ __global__ __launch_bounds__(NT) void latent_attn_k(
       __syncthreads();
       for (int i = tid; i < nk * D; i += NT) {
         const int kk = i / D, c = i - kk * D;
-        const int p = k0 + kk;
+        const int p = klo + k0 + kk;
         const int64_t r = (int64_t)tab[p / bs] * bs + p % bs;
         ks[kk * DS + c] = pool[r * D + c];
       }
@@ -201,7 +217,13 @@ __global__ __launch_bounds__(NT) void latent_attn_k(
     for (int h = 0; h < HG; ++h) {
       if (h < nh) {
         if (nsplit == 1) {
-          const float inv = 1.f / lrun[h];
+          float inv = 1.f / lrun[h];
+          if (sink) {  // one more term of the denominator, no value
+            const float sk = sink[h0 + h];
+            const float m2 = fmaxf(mrun[h], sk);
+            const float f = expf(mrun[h] - m2);
+            inv = f / (lrun[h] * f + expf(sk - m2));
+          }
 #pragma unroll
           for (int i = 0; i < RPT; ++i) {
             const int col = tid + i * NT;
@@ -228,12 +250,12 @@ __global__ __launch_bounds__(NT) void latent_attn_k(
 template <typename T>
 __global__ __launch_bounds__(NT) void latent_attn_merge_k(
     const float* __restrict__ part, T* __restrict__ out, int Ttok, int H,
-    int rank, int nsplit) {
+    int rank, int nsplit, const float* __restrict__ sink) {
   const int t = blockIdx.x, h = blockIdx.y;
-  float m = -INFINITY;
+  float m = sink ? sink[h] : -INFINITY;
   for (int s = 0; s < nsplit; ++s)
     m = fmaxf(m, part[(((int64_t)t * nsplit + s) * H + h) * (rank + 2)]);
-  float l = 0.f;
+  float l = sink ? expf(sink[h] - m) : 0.f;
   for (int s = 0; s < nsplit; ++s) {
     const float* pp = part + (((int64_t)t * nsplit + s) * H + h) * (rank + 2);
     if (pp[1] > 0.f) l += pp[1] * expf(pp[0] - m);
@@ -280,7 +302,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
     const int* __restrict__ cu, const int* __restrict__ seq_start,
     const int* __restrict__ table, int maxb, int bs, bf16* __restrict__ out,
     float* __restrict__ part,  // [Ttok, nsplit, H, rank + 2] when nsplit > 1
-    int Ttok, int H, int rank, int rot, int nsplit, float scale) {
+    int Ttok, int H, int rank, int rot, int nsplit, float scale, int window,
+    const float* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   constexpr int DVW = DVB / SPLIT;     // output blocks of this wave
   constexpr int ROWS = TB_ROWS / SPLIT;
@@ -307,10 +330,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
   const int qpos = start + j;
   const int kmax = start + min(m0 + ROWS - 1, rows - 1) / H;  // inclusive
   const int* tab = table + (int64_t)s * maxb;
+  // first key this row sees, and the tile's earliest (its first row's)
+  const int klo = window > 0 ? max(0, qpos - window + 1) : 0;
+  const int kmin = window > 0 ? max(0, start + m0 / H - window + 1) : 0;
   // this split's key steps
-  const int nsteps = kmax / TB_KEYS + 1;
+  const int step0 = kmin / TB_KEYS;
+  const int nsteps = kmax / TB_KEYS + 1 - step0;
   const int per = (nsteps + nsplit - 1) / nsplit;
-  const int s_lo = split * per, s_hi = min(nsteps, s_lo + per);
+  const int s_lo = step0 + split * per, s_hi = min(step0 + nsteps, s_lo + per);
   float* pp = nullptr;
   if (nsplit > 1)
     pp = part + (((int64_t)t * nsplit + split) * H + h) * (rank + 2);
@@ -463,7 +490,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int key = k0 + (r & 3) + 8 * (r >> 2) + 4 * hl;
-      const float v = key <= qpos ? st[r] * scale : -INFINITY;
+      const float v = (key <= qpos && key >= klo) ? st[r] * scale : -INFINITY;
       st[r] = v;
       mx = fmaxf(mx, v);
     }
@@ -526,7 +553,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
           if (d < rank) pp[2 + d] = oacc[db][r];
         }
     } else {
-      const float inv = 1.f / lrun;
+      float inv = 1.f / lrun;
+      if (sink) {  // one more term of the denominator, no value
+        const float sk = sink[h];
+        const float m2 = fmaxf(mrun, sk);
+        const float f = __expf(mrun - m2);
+        inv = f / (lrun * f + __expf(sk - m2));
+      }
       bf16* o = out + ((int64_t)h * Ttok + t) * rank;
 #pragma unroll
       for (int db = 0; db < DVW; ++db)
@@ -544,7 +577,7 @@ int launch_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* po
                             const int* work, int nwork, const int* cu, const int* seq_start,
                             const int* table, int maxb, int bs, void* out, float* part,
                             int Ttok, int H, int rank, int rot, int nsplit, float scale,
-                            hipStream_t s) {
+                            int window, const float* sink, hipStream_t s) {
   const int DkP = (rank + rot + 15) & ~15;
   const size_t lds = (size_t)TB_KEYS * (DkP + 8) * 2 + (size_t)DVB * 32 * VT_STRIDE * 2 +
                      (SPLIT == 2 ? 4 * 16 * 64 * 4 : 0);
@@ -557,13 +590,14 @@ int launch_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* po
   kern<<<dim3(nwork, nsplit), 256, lds, s>>>((const short*)q_lat, (const short*)q_rot,
                                              (const short*)pool, work, cu, seq_start, table, maxb,
                                              bs, (bf16*)out, part, Ttok, H, rank, rot, nsplit,
-                                             scale);
+                                             scale, window, sink);
   if (nsplit > 1)
-    latent_attn_merge_k<bf16><<<dim3(Ttok, H), NT, 0, s>>>(part, (bf16*)out, Ttok, H, rank, nsplit);
+    latent_attn_merge_k<bf16><<<dim3(Ttok, H), NT, 0, s>>>(part, (bf16*)out, Ttok, H, rank, nsplit,
+                                                           sink);
   return (int)hipGetLastError();
 }
 
-// out[t, h*v + c] = o[h, t, c] * gate[t, h]
+// out[t, h*v + c] = o[h, t, c] * gate[t, h] (gate null: heads merged as they are)
 template <typename T>
 __global__ void gate_merge_k(const T* __restrict__ o, const float* __restrict__ gate,
                              T* __restrict__ out, int Ttok, int H, int v) {
@@ -573,7 +607,7 @@ __global__ void gate_merge_k(const T* __restrict__ o, const float* __restrict__ 
     const int c = i % v;
     const int h = (i / v) % H;
     const int64_t t = i / ((int64_t)v * H);
-    st(out + i, ld(o + ((int64_t)h * Ttok + t) * v + c) * gate[t * H + h]);
+    st(out + i, ld(o + ((int64_t)h * Ttok + t) * v + c) * (gate ? gate[t * H + h] : 1.f));
   }
 }
 
@@ -581,14 +615,19 @@ __global__ void gate_merge_k(const T* __restrict__ o, const float* __restrict__ 
 
 extern "C" {
 
-int dsv_latent_prep(const void* proj, int ld_proj, const float* norm_w, const int* tok_pos,
+int dsv_latent_prep(const void* q_src, int ld_q, const void* kv_src, int ld_kv,
+                    const void* gate_src, int ld_g, const float* norm_w, const int* tok_pos,
                     const int* tok_row, const float* cosT, const float* sinT, void* pool,
                     void* q_nope, void* q_rot, float* gate, int dt, int Ttok, int H, int dim,
-                    int rot, int rank, int rot_dims, float eps, hipStream_t s) {
+                    int rot, int rank, int rot_dims, float eps, int half_layout, hipStream_t s) {
   if (Ttok <= 0) return 0;
+  if (rot_dims < 0 || rot_dims > rot || (rot_dims & 1)) return -1;
+  if (rot_dims && (!cosT || !sinT)) return -2;
+  if (gate_src && !gate) return -3;
   BY_DTYPE(dt, (latent_prep_k<T><<<Ttok, NT, 0, s>>>(
-                   (const T*)proj, ld_proj, norm_w, tok_pos, tok_row, cosT, sinT, (T*)pool,
-                   (T*)q_nope, (T*)q_rot, gate, Ttok, H, dim, rot, rank, rot_dims, eps)));
+                   (const T*)q_src, ld_q, (const T*)kv_src, ld_kv, (const T*)gate_src, ld_g,
+                   norm_w, tok_pos, tok_row, cosT, sinT, (T*)pool, (T*)q_nope, (T*)q_rot, gate,
+                   Ttok, H, dim, rot, rank, rot_dims, eps, half_layout)));
   return (int)hipGetLastError();
 }
 
@@ -601,18 +640,20 @@ int64_t dsv_latent_attn_lds(int dt, int rank, int rot, int KC) {
 int dsv_latent_attn(const void* q_lat, const void* q_rot, const void* pool, const int* tok_seq,
                     const int* tok_pos, const int* table, int maxb, int bs, void* out,
                     float* part, int dt, int Ttok, int H, int rank, int rot, int KC,
-                    int nsplit, float scale, hipStream_t s) {
-  if (rank > RPT * NT) return -1;
+                    int nsplit, float scale, int window, const float* sink, hipStream_t s) {
+  if (rank > RPT * NT || window < 0) return -1;
   if (Ttok <= 0) return 0;
   const int64_t lds = dsv_latent_attn_lds(dt, rank, rot, KC);
   if (lds > 64 * 1024) return -2;
   dim3 grid(Ttok, nsplit);
   BY_DTYPE(dt, (latent_attn_k<T><<<grid, NT, lds, s>>>(
                    (const T*)q_lat, (const T*)q_rot, (const T*)pool, tok_seq, tok_pos, table,
-                   maxb, bs, (T*)out, part, Ttok, H, rank, rot, KC, nsplit, scale)));
+                   maxb, bs, (T*)out, part, Ttok, H, rank, rot, KC, nsplit, scale, window,
+                   sink)));
   if (nsplit > 1) {
     dim3 g2(Ttok, H);
-    BY_DTYPE(dt, (latent_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, Ttok, H, rank, nsplit)));
+    BY_DTYPE(dt, (latent_attn_merge_k<T><<<g2, NT, 0, s>>>(part, (T*)out, Ttok, H, rank, nsplit,
+                                                           sink)));
   }
   return (int)hipGetLastError();
 }
@@ -631,15 +672,16 @@ int dsv_latent_attn_mfma_rows(int rank, int rot) {
 int dsv_latent_attn_mfma(const void* q_lat, const void* q_rot, const void* pool, const int* work,
                          int nwork, const int* cu, const int* seq_start, const int* table,
                          int maxb, int bs, void* out, float* part, int Ttok, int H, int rank,
-                         int rot, int nsplit, float scale, hipStream_t s) {
-  if (!dsv_latent_attn_mfma_ok(rank, rot)) return -1;
+                         int rot, int nsplit, float scale, int window, const float* sink,
+                         hipStream_t s) {
+  if (!dsv_latent_attn_mfma_ok(rank, rot) || window < 0) return -1;
   if (nsplit < 1 || (nsplit > 1 && !part)) return -3;
   if (nwork <= 0) return 0;
   const int dk = rank + rot;
 #define GO(DVB, DKT, SPLIT, PF) \
   return launch_latent_attn_mfma<DVB, DKT, SPLIT, PF>(q_lat, q_rot, pool, work, nwork, cu, seq_start, \
                                            table, maxb, bs, out, part, Ttok, H, rank, rot, \
-                                           nsplit, scale, s)
+                                           nsplit, scale, window, sink, s)
   if (rank <= 64 && dk <= 128) GO(2, 8, 1, true);
   if (rank <= 128 && dk <= 192) GO(4, 12, 1, true);
   if (rank <= 256 && dk <= 320) GO(8, 20, 1, true);

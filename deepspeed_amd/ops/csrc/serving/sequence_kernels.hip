@@ -698,7 +698,9 @@ int launch_window_attn_mfma(const void* q, const void* pool, const int* work, in
 }
 
 // -------------------------------------------------- delta-rule prologue
-// proj row = [ q (G x dim) | k (G x dim) | v (H x vdim) | gate | b (H) | a (H) ].
+// proj row = [ q (G x dim) | k (G x dim) | v (H x vdim) | ... ]; the H columns
+// of b start at beta_col and those of a at a_col (a_col < 0: the decay is not
+// made here, e.g. one per key channel that comes from a product of its own).
 // One block per token: causal convolution + SiLU over the q|k|v channels
 // (earlier inputs from this step's rows, from the slot's tail, or zero before
 // position 0), q and k to unit length per head (q also times dim^-1/2),
@@ -713,7 +715,7 @@ __global__ __launch_bounds__(NT) void delta_prep_k(
     const int* __restrict__ tok_pos, const float* __restrict__ a_log,
     const float* __restrict__ dt_bias, float* __restrict__ q_out, float* __restrict__ k_out,
     float* __restrict__ v_out, float* __restrict__ beta, float* __restrict__ decay, int G, int H,
-    int dim, int vdim, int taps) {
+    int dim, int vdim, int taps, int beta_col, int a_col) {
   extern __shared__ float ys[];  // [2*G*dim] conv outputs of q and k
   const int t = blockIdx.x;
   const int s = tok_seq[t];
@@ -752,9 +754,11 @@ __global__ __launch_bounds__(NT) void delta_prep_k(
     for (int c = lane; c < dim; c += 64) o[c] = y[c] * inv;
   }
   for (int h = threadIdx.x; h < H; h += NT) {
-    beta[(int64_t)t * H + h] = sigmoidf_(ld(p + C + nv + h));
-    const float dt = softplusf_(ld(p + C + nv + H + h) + dt_bias[h]);
-    decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * dt);
+    beta[(int64_t)t * H + h] = sigmoidf_(ld(p + beta_col + h));
+    if (a_col >= 0) {
+      const float dt = softplusf_(ld(p + a_col + h) + dt_bias[h]);
+      decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * dt);
+    }
   }
 }
 
@@ -767,7 +771,7 @@ __global__ __launch_bounds__(NT) void delta_prep_vec_k(
     const int* __restrict__ tok_pos, const float* __restrict__ a_log,
     const float* __restrict__ dt_bias, float* __restrict__ q_out, float* __restrict__ k_out,
     float* __restrict__ v_out, float* __restrict__ beta, float* __restrict__ decay, int G, int H,
-    int dim, int vdim) {
+    int dim, int vdim, int beta_col, int a_col) {
   extern __shared__ float ys[];  // [2*G*dim] conv outputs of q and k
   constexpr int TAIL = TAPS - 1;
   const int t = blockIdx.x;
@@ -823,9 +827,11 @@ __global__ __launch_bounds__(NT) void delta_prep_vec_k(
     for (int c = lane; c < dim; c += 64) o[c] = y[c] * inv;
   }
   for (int h = threadIdx.x; h < H; h += NT) {
-    beta[(int64_t)t * H + h] = sigmoidf_(ld(p + C + nv + h));
-    const float dt = softplusf_(ld(p + C + nv + H + h) + dt_bias[h]);
-    decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * dt);
+    beta[(int64_t)t * H + h] = sigmoidf_(ld(p + beta_col + h));
+    if (a_col >= 0) {
+      const float dt = softplusf_(ld(p + a_col + h) + dt_bias[h]);
+      decay[(int64_t)t * H + h] = expf(-expf(a_log[h]) * dt);
+    }
   }
 }
 
@@ -865,6 +871,23 @@ __global__ void sigmoid_pow_k(const T* __restrict__ z, const float* __restrict__
     const float x = ld(z + i) + bias[i % C];
     const float ls = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
     out[i] = expf(inv_tau * ls);
+  }
+}
+
+// exp(-exp(a_log[h]) * softplus(z + bias)) per head h and key channel: z is
+// [rows, H*dim] with row stride ld_z, bias [H*dim], out [rows, H, dim] float.
+template <typename T>
+__global__ void softplus_decay_k(const T* __restrict__ z, int ld_z, const float* __restrict__ bias,
+                                 const float* __restrict__ a_log, float* __restrict__ out,
+                                 int64_t rows, int H, int dim) {
+  const int C = H * dim;
+  const int64_t n = rows * C;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / C;
+    const int c = (int)(i - r * C);
+    const float dt = softplusf_(ld(z + r * ld_z + c) + bias[c]);
+    out[i] = expf(-expf(a_log[c / dim]) * dt);
   }
 }
 
@@ -1115,8 +1138,9 @@ __global__ __launch_bounds__(NT) void linear_scan_k(
   }
 }
 
-// out[t, h*vdim + c] = o / sqrt(mean_c(o^2) + eps) * w[c] * silu(gate)
-template <typename T>
+// out[t, h*vdim + c] = o / sqrt(mean_c(o^2) + eps) * w[c] * act(gate),
+// act = SiLU, or the plain sigmoid with SIGMOID
+template <typename T, bool SIGMOID>
 __global__ __launch_bounds__(NT) void head_norm_gate_k(
     const float* __restrict__ o, const float* __restrict__ w, const T* __restrict__ gate,
     int ld_gate, T* __restrict__ out, int H, int vdim, float eps) {
@@ -1129,7 +1153,8 @@ __global__ __launch_bounds__(NT) void head_norm_gate_k(
     const float inv = rsqrtf(wave_sum(ss) / (float)vdim + eps);
     for (int c = lane; c < vdim; c += 64) {
       const float gv = ld(gate + (int64_t)t * ld_gate + h * vdim + c);
-      st(out + ((int64_t)t * H + h) * vdim + c, oh[c] * inv * w[c] * siluf_(gv));
+      st(out + ((int64_t)t * H + h) * vdim + c,
+         oh[c] * inv * w[c] * (SIGMOID ? sigmoidf_(gv) : siluf_(gv)));
     }
   }
 }
@@ -1772,8 +1797,10 @@ int dsv_delta_prep(const void* proj, int ld_proj, const void* w, void* state,
                    const int* seq_start, const int* tok_seq, const int* tok_pos,
                    const float* a_log, const float* dt_bias, float* q_out, float* k_out,
                    float* v_out, float* beta, float* decay, int dt, int Ttok, int nseq, int G,
-                   int H, int dim, int vdim, int taps, hipStream_t s) {
+                   int H, int dim, int vdim, int taps, int beta_col, int a_col, hipStream_t s) {
   if (taps < 1 || taps > MAXTAPS_SEQ || H % G) return -1;
+  if (beta_col < 0 || beta_col + H > ld_proj || a_col + H > ld_proj) return -3;
+  if (a_col >= 0 && !decay) return -3;
   if (Ttok <= 0) return 0;
   const int64_t lds = (int64_t)2 * G * dim * 4;
   if (lds > 64 * 1024) return -2;
@@ -1785,7 +1812,7 @@ int dsv_delta_prep(const void* proj, int ld_proj, const void* w, void* state,
   BY_DTYPE(dt, (delta_prep_vec_k<T, TAPS><<<Ttok, NT, lds, s>>>(                                \
                    (const T*)proj, ld_proj, (const T*)w, (const T*)state, state_slot_stride,   \
                    cu, seq_slot, tok_seq, tok_pos, a_log, dt_bias, q_out, k_out, v_out, beta,  \
-                   decay, G, H, dim, vdim)))
+                   decay, G, H, dim, vdim, beta_col, a_col)))
   if (vec && taps == 4)
     PREP_VEC(4);
   else if (vec && taps == 2)
@@ -1795,7 +1822,7 @@ int dsv_delta_prep(const void* proj, int ld_proj, const void* w, void* state,
   BY_DTYPE(dt, (delta_prep_k<T><<<Ttok, NT, lds, s>>>(
                    (const T*)proj, ld_proj, (const T*)w, (const T*)state, state_slot_stride, cu,
                    seq_slot, tok_seq, tok_pos, a_log, dt_bias, q_out, k_out, v_out, beta, decay,
-                   G, H, dim, vdim, taps)));
+                   G, H, dim, vdim, taps, beta_col, a_col)));
   if (taps > 1)
     BY_DTYPE(dt, (conv_tail_shift_k<T><<<nseq, NT, 0, s>>>((const T*)proj, ld_proj, (T*)state,
                                                            state_slot_stride, cu, seq_slot,
@@ -1842,11 +1869,26 @@ int dsv_linear_scan(const void* q, int ld_q, const void* k, int ld_k, const void
   return (int)hipGetLastError();
 }
 
+// act: 0 = SiLU of the gate, 1 = sigmoid
 int dsv_head_norm_gate(const float* o, const float* w, const void* gate, int ld_gate, void* out,
-                       int dt, int Ttok, int H, int vdim, float eps, hipStream_t s) {
+                       int dt, int Ttok, int H, int vdim, float eps, int act, hipStream_t s) {
   if (Ttok <= 0) return 0;
-  BY_DTYPE(dt, (head_norm_gate_k<T><<<Ttok, NT, 0, s>>>(o, w, (const T*)gate, ld_gate, (T*)out, H,
-                                                        vdim, eps)));
+  if (act == 1)
+    BY_DTYPE(dt, (head_norm_gate_k<T, true><<<Ttok, NT, 0, s>>>(o, w, (const T*)gate, ld_gate,
+                                                                (T*)out, H, vdim, eps)));
+  else if (act == 0)
+    BY_DTYPE(dt, (head_norm_gate_k<T, false><<<Ttok, NT, 0, s>>>(o, w, (const T*)gate, ld_gate,
+                                                                 (T*)out, H, vdim, eps)));
+  else
+    return -1;
+  return (int)hipGetLastError();
+}
+
+int dsv_softplus_decay(const void* z, int ld_z, const float* bias, const float* a_log, float* out,
+                       int dt, int64_t rows, int H, int dim, hipStream_t s) {
+  if (rows * H * dim <= 0) return 0;
+  BY_DTYPE(dt, (softplus_decay_k<T><<<nblocks(rows * H * dim, 256), 256, 0, s>>>(
+                   (const T*)z, ld_z, bias, a_log, out, rows, H, dim)));
   return (int)hipGetLastError();
 }
 

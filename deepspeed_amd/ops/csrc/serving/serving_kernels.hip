@@ -125,14 +125,46 @@ __global__ __launch_bounds__(NT) void layer_norm_vec_k(
   }
 }
 
-// out[r] = table[ids[r]] * scale (fp32)
+// out[r] = table[ids[r]] * scale (+ table2[ids2[r]]) (fp32)
 template <typename T>
 __global__ __launch_bounds__(NT) void embed_rows_k(
-    const T* __restrict__ table, const int64_t* __restrict__ ids, float* __restrict__ out,
-    int C, float scale) {
+    const T* __restrict__ table, const int64_t* __restrict__ ids, const T* __restrict__ table2,
+    const int64_t* __restrict__ ids2, float* __restrict__ out, int C, float scale) {
   const int64_t r = blockIdx.x;
   const T* row = table + ids[r] * (int64_t)C;
-  for (int c = threadIdx.x; c < C; c += NT) out[r * C + c] = ld(row + c) * scale;
+  const T* row2 = table2 ? table2 + ids2[r] * (int64_t)C : nullptr;
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float v = ld(row + c) * scale;
+    if (row2) v += ld(row2 + c);
+    out[r * C + c] = v;
+  }
+}
+
+// Row of a hashed pair table for every token of a ragged step:
+// (previous * mul_prev + current * mul_cur) mod buckets, and row `buckets` for
+// a sequence's first token. The previous token of a step's first token is the
+// slot's carried one. pair_hash_tail_k then stores each sequence's last token
+// (a launch of its own: every read of the old value has finished).
+__global__ void pair_hash_rows_k(const int64_t* __restrict__ ids, const int* __restrict__ cu,
+                                 const int* __restrict__ seq_slot, const int* __restrict__ tok_seq,
+                                 const int* __restrict__ tok_pos, const int64_t* __restrict__ prev,
+                                 int64_t* __restrict__ rows, int Ttok, int64_t mul_prev,
+                                 int64_t mul_cur, int64_t buckets) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= Ttok) return;
+  if (tok_pos[t] == 0) {
+    rows[t] = buckets;
+    return;
+  }
+  const int s = tok_seq[t];
+  const int64_t before = t > cu[s] ? ids[t - 1] : prev[seq_slot[s]];
+  rows[t] = (before * mul_prev + ids[t] * mul_cur) % buckets;
+}
+__global__ void pair_hash_tail_k(const int64_t* __restrict__ ids, const int* __restrict__ cu,
+                                 const int* __restrict__ seq_slot, int64_t* __restrict__ prev,
+                                 int nseq) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s < nseq && cu[s + 1] > cu[s]) prev[seq_slot[s]] = ids[cu[s + 1] - 1];
 }
 
 // ------------------------------------------------- norm + causal conv
@@ -481,25 +513,41 @@ __global__ void glu8_k(const T* __restrict__ gu, T* __restrict__ out, int64_t ro
   }
 }
 
-// Per token: scores s = sigmoid(z); choice c = s + corr. Experts form `groups`
-// equal runs; a group's score is the sum of its two largest c (its one when
-// a run holds one expert); only experts of the `keep` best groups compete.
-// The `top` largest allowed c are chosen; weights are their s.
+// Per token: scores s = sigmoid(z), or softmax(z) over all E with SOFTMAX;
+// choice c = s + corr. Experts form `groups` equal runs; a group's score is the
+// sum of its two largest c (its one when a run holds one expert), or its
+// largest alone with `group_max`; only experts of the `keep` best groups
+// compete (the others count as minus infinity: c may be negative). The `top`
+// largest allowed c are chosen; weights are their s, with `renorm` divided by
+// their sum (+ 1e-20), times `scale`.
 constexpr int MAXGROUPS = 64;
-__global__ void grouped_sigmoid_topk_k(const float* __restrict__ z, const float* __restrict__ corr,
-                                       int64_t* __restrict__ idx, float* __restrict__ w,
-                                       int Ttok, int E, int top, int groups, int keep) {
+template <bool SOFTMAX>
+__global__ void grouped_topk_k(const float* __restrict__ z, const float* __restrict__ corr,
+                               int64_t* __restrict__ idx, float* __restrict__ w, int Ttok, int E,
+                               int top, int groups, int keep, int group_max, int renorm,
+                               float scale) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= Ttok) return;
   const float* r = z + (int64_t)t * E;
   const int per = E / groups;
+  float zmax = 0.f, zinv = 1.f;
+  if (SOFTMAX) {
+    zmax = -INFINITY;
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, r[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) sum += expf(r[e] - zmax);
+    zinv = 1.f / sum;
+  }
+  auto score = [&](int e) -> float {
+    return SOFTMAX ? expf(r[e] - zmax) * zinv : 1.f / (1.f + expf(-r[e]));
+  };
   unsigned long long allowed = ~0ull;
   if (groups > 1) {
     float gs[MAXGROUPS];
     for (int g = 0; g < groups; ++g) {
       float a = -INFINITY, b2 = -INFINITY;  // largest, second largest
       for (int e = g * per; e < (g + 1) * per; ++e) {
-        const float c = 1.f / (1.f + expf(-r[e])) + corr[e];
+        const float c = score(e) + corr[e];
         if (c > a) {
           b2 = a;
           a = c;
@@ -507,7 +555,7 @@ __global__ void grouped_sigmoid_topk_k(const float* __restrict__ z, const float*
           b2 = c;
         }
       }
-      gs[g] = per > 1 ? a + b2 : a;
+      gs[g] = (per > 1 && !group_max) ? a + b2 : a;
     }
     allowed = 0ull;
     for (int k = 0; k < keep; ++k) {
@@ -521,6 +569,7 @@ __global__ void grouped_sigmoid_topk_k(const float* __restrict__ z, const float*
       allowed |= 1ull << bi;
     }
   }
+  float total = 0.f;
   for (int k = 0; k < top; ++k) {
     int bi = -1;
     float bv = -INFINITY, bs = 0.f;
@@ -529,7 +578,7 @@ __global__ void grouped_sigmoid_topk_k(const float* __restrict__ z, const float*
       bool taken = false;
       for (int q = 0; q < k; ++q) taken |= idx[(int64_t)t * top + q] == e;
       if (taken) continue;
-      const float sg = 1.f / (1.f + expf(-r[e]));
+      const float sg = score(e);
       const float c = sg + corr[e];
       if (bi < 0 || c > bv) {
         bi = e;
@@ -539,7 +588,11 @@ __global__ void grouped_sigmoid_topk_k(const float* __restrict__ z, const float*
     }
     idx[(int64_t)t * top + k] = bi;
     w[(int64_t)t * top + k] = bs;
+    total += bs;
   }
+  const float f = renorm ? scale / (total + 1e-20f) : scale;
+  if (renorm || scale != 1.f)
+    for (int k = 0; k < top; ++k) w[(int64_t)t * top + k] *= f;
 }
 
 // out[t] = sum_k w[t,k] * y[inv[t,k]] (+ sigmoid(sg[t]) * shared[t])
@@ -588,15 +641,16 @@ __global__ void topk_softmax_k(const float* __restrict__ z, int64_t* __restrict_
 
 
 // ------------------------------------------------ weighted RMS norm of rows
-// out[r] = x[idx ? idx[r] : r] / sqrt(mean(x^2) + eps) * (w or 1 + w); the
-// VEC form keeps the row in registers (C a multiple of 8, at most 8*NT*LN_G).
+// out[r] = x[idx ? idx[r] : r] / sqrt(mean(x^2) + eps) * (w or 1 + w); input
+// rows may be a column slice (row stride ld_in). The VEC form keeps the row in
+// registers (C a multiple of 8, at most 8*NT*LN_G).
 template <typename TI, typename TO, bool VEC>
 __global__ __launch_bounds__(NT) void rms_norm_rows_k(
-    const TI* __restrict__ in, const int64_t* __restrict__ idx, const float* __restrict__ w,
-    TO* __restrict__ out, int C, float eps, float w_add) {
+    const TI* __restrict__ in, int ld_in, const int64_t* __restrict__ idx,
+    const float* __restrict__ w, TO* __restrict__ out, int C, float eps, float w_add) {
   __shared__ float red[NT / 64];
   const int64_t r = blockIdx.x;
-  const TI* row = in + (idx ? idx[r] : r) * (int64_t)C;
+  const TI* row = in + (idx ? idx[r] : r) * (int64_t)ld_in;
   TO* o = out + r * (int64_t)C;
   if (VEC) {
     float v[LN_G][8];
@@ -707,6 +761,100 @@ __global__ __launch_bounds__(NT) void gated_add_k(
     if (!w) return;
     const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
     for (int c = threadIdx.x; c < C; c += NT) st(h + r * C + c, xr[c] * inv * (w[c] + w_add));
+  }
+}
+
+// ------------------------------------- scaled residual add, paired norms
+// x[r] += s1 * y1[r] (+ s2 * y2[r]) (+ extra[r]) on the float stream, s1/s2 one
+// factor per column (y1 may be null: nothing is added, the row is only normed).
+// With w1 (and w2) the same pass emits the RMS norm of the new row under each
+// weight: two sublayers that read the same row through norms of their own
+// share one read and one statistic.
+template <typename T, typename TO, bool VEC>
+__global__ __launch_bounds__(NT) void scaled_add_k(
+    float* __restrict__ x, const float* __restrict__ s1, const T* __restrict__ y1,
+    const float* __restrict__ s2, const T* __restrict__ y2, const float* __restrict__ extra,
+    const float* __restrict__ w1, const float* __restrict__ w2, TO* __restrict__ h1,
+    TO* __restrict__ h2, int C, float eps) {
+  __shared__ float red[NT / 64];
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * C;
+  const T* b1 = y1 ? y1 + r * C : nullptr;
+  const T* b2 = y2 ? y2 + r * C : nullptr;
+  const float* ex = extra ? extra + r * C : nullptr;
+  if (VEC) {
+    float v[LN_G][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_G; ++i) {
+      const int c = (threadIdx.x + i * NT) * 8;
+      if (c < C) {
+        load8(xr + c, v[i]);
+        if (b1) {
+          float d[8], y[8], sc[8];
+          load8(b1 + c, y);
+          load8(s1 + c, sc);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) d[e] = sc[e] * y[e];
+          if (b2) {
+            load8(b2 + c, y);
+            load8(s2 + c, sc);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d[e] += sc[e] * y[e];
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] += d[e];
+        }
+        if (ex) {
+          float y[8];
+          load8(ex + c, y);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[i][e] += y[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+        if (b1 || ex) store8(xr + c, v[i]);
+      }
+    }
+    if (!w1) return;
+    const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+#pragma unroll
+    for (int i = 0; i < LN_G; ++i) {
+      const int c = (threadIdx.x + i * NT) * 8;
+      if (c < C) {
+        float wv[8], o[8];
+        load8(w1 + c, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = v[i][e] * inv * wv[e];
+        store8(h1 + r * C + c, o);
+        if (w2) {
+          load8(w2 + c, wv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] = v[i][e] * inv * wv[e];
+          store8(h2 + r * C + c, o);
+        }
+      }
+    }
+  } else {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < C; c += NT) {
+      float v = xr[c];
+      if (b1) {
+        float d = s1[c] * ld(b1 + c);
+        if (b2) d += s2[c] * ld(b2 + c);
+        v += d;
+      }
+      if (ex) v += ex[c];
+      if (b1 || ex) xr[c] = v;
+      ss += v * v;
+    }
+    if (!w1) return;
+    const float inv = rsqrtf(block_sum(ss, red) / (float)C + eps);
+    for (int c = threadIdx.x; c < C; c += NT) {
+      const float v = xr[c] * inv;
+      st(h1 + r * C + c, v * w1[c]);
+      if (w2) st(h2 + r * C + c, v * w2[c]);
+    }
   }
 }
 
@@ -848,10 +996,23 @@ int dsv_layer_norm(const void* in, int in_dt, const int64_t* idx, const float* w
   return (int)hipGetLastError();
 }
 
-int dsv_embed_rows(const void* table, int dt, const int64_t* ids, float* out, int rows, int C,
-                   float scale, hipStream_t s) {
+int dsv_embed_rows(const void* table, int dt, const int64_t* ids, const void* table2,
+                   const int64_t* ids2, float* out, int rows, int C, float scale, hipStream_t s) {
   if (rows <= 0) return 0;
-  BY_DTYPE(dt, (embed_rows_k<T><<<rows, NT, 0, s>>>((const T*)table, ids, out, C, scale)));
+  if ((table2 == nullptr) != (ids2 == nullptr)) return -1;
+  BY_DTYPE(dt, (embed_rows_k<T><<<rows, NT, 0, s>>>((const T*)table, ids, (const T*)table2, ids2,
+                                                    out, C, scale)));
+  return (int)hipGetLastError();
+}
+
+int dsv_pair_hash_rows(const int64_t* ids, const int* cu, const int* seq_slot, const int* tok_seq,
+                       const int* tok_pos, int64_t* prev, int64_t* rows, int Ttok, int nseq,
+                       int64_t mul_prev, int64_t mul_cur, int64_t buckets, hipStream_t s) {
+  if (buckets < 1 || mul_prev < 0 || mul_cur < 0) return -1;
+  if (Ttok <= 0) return 0;
+  pair_hash_rows_k<<<(Ttok + 255) / 256, 256, 0, s>>>(ids, cu, seq_slot, tok_seq, tok_pos, prev,
+                                                      rows, Ttok, mul_prev, mul_cur, buckets);
+  pair_hash_tail_k<<<(nseq + 63) / 64, 64, 0, s>>>(ids, cu, seq_slot, prev, nseq);
   return (int)hipGetLastError();
 }
 
@@ -876,13 +1037,26 @@ int dsv_glu(const void* gu, void* out, int dt, int64_t rows, int F, int act, hip
   return (int)hipGetLastError();
 }
 
-int dsv_grouped_sigmoid_topk(const float* z, const float* corr, int64_t* idx, float* w, int Ttok,
-                             int E, int top, int groups, int keep, hipStream_t s) {
+// kind: 0 = sigmoid scores, 1 = softmax over all experts
+int dsv_grouped_topk(const float* z, const float* corr, int64_t* idx, float* w, int Ttok, int E,
+                     int top, int groups, int keep, int kind, int group_max, int renorm,
+                     float scale, hipStream_t s) {
   if (groups < 1 || groups > MAXGROUPS || E % groups || keep < 1 || keep > groups) return -1;
   if (top < 1 || top > keep * (E / groups)) return -2;
+  if (kind != 0 && kind != 1) return -3;
   if (Ttok <= 0) return 0;
-  grouped_sigmoid_topk_k<<<(Ttok + 63) / 64, 64, 0, s>>>(z, corr, idx, w, Ttok, E, top, groups, keep);
+  if (kind == 1)
+    grouped_topk_k<true><<<(Ttok + 63) / 64, 64, 0, s>>>(z, corr, idx, w, Ttok, E, top, groups,
+                                                         keep, group_max, renorm, scale);
+  else
+    grouped_topk_k<false><<<(Ttok + 63) / 64, 64, 0, s>>>(z, corr, idx, w, Ttok, E, top, groups,
+                                                          keep, group_max, renorm, scale);
   return (int)hipGetLastError();
+}
+
+int dsv_grouped_sigmoid_topk(const float* z, const float* corr, int64_t* idx, float* w, int Ttok,
+                             int E, int top, int groups, int keep, hipStream_t s) {
+  return dsv_grouped_topk(z, corr, idx, w, Ttok, E, top, groups, keep, 0, 0, 0, 1.f, s);
 }
 
 int dsv_xielu(const void* z, const float* pq, void* out, int dt, int64_t n, hipStream_t s) {
@@ -913,19 +1087,22 @@ int dsv_topk_softmax(const float* z, int64_t* idx, float* w, int Ttok, int E, in
   return (int)hipGetLastError();
 }
 
-int dsv_rms_norm_rows(const void* x, int in_dt, const int64_t* idx, const float* w, void* out,
-                      int out_dt, int rows, int C, float eps, int one_plus, hipStream_t s) {
+int dsv_rms_norm_rows(const void* x, int in_dt, int ld_in, const int64_t* idx, const float* w,
+                      void* out, int out_dt, int rows, int C, float eps, int one_plus,
+                      hipStream_t s) {
   if (rows <= 0) return 0;
+  if (ld_in < C) return -1;
   const float wa = one_plus ? 1.f : 0.f;
-  const bool vec = C % 8 == 0 && C <= 8 * NT * LN_G;
+  const bool vec = C % 8 == 0 && C <= 8 * NT * LN_G && ld_in % 8 == 0 &&
+                   (uintptr_t)x % 32 == 0;
 #define RN(TI, TO)                                                                              \
   do {                                                                                          \
     if (vec)                                                                                    \
-      rms_norm_rows_k<TI, TO, true><<<rows, NT, 0, s>>>((const TI*)x, idx, w, (TO*)out, C, eps, \
-                                                        wa);                                    \
+      rms_norm_rows_k<TI, TO, true><<<rows, NT, 0, s>>>((const TI*)x, ld_in, idx, w, (TO*)out,  \
+                                                        C, eps, wa);                            \
     else                                                                                        \
-      rms_norm_rows_k<TI, TO, false><<<rows, NT, 0, s>>>((const TI*)x, idx, w, (TO*)out, C,     \
-                                                         eps, wa);                              \
+      rms_norm_rows_k<TI, TO, false><<<rows, NT, 0, s>>>((const TI*)x, ld_in, idx, w, (TO*)out, \
+                                                         C, eps, wa);                           \
   } while (0)
   if (in_dt == 0 && out_dt == 0) RN(float, float);
   else if (in_dt == 0) RN(float, bf16);
@@ -961,6 +1138,31 @@ int dsv_gated_add(float* x, const void* g1, const void* g2, int ld_g, const void
   else if (out_dt == 0) GA(bf16, float);
   else GA(bf16, bf16);
 #undef GA
+  return (int)hipGetLastError();
+}
+
+// y1/y2 (dtype dt) may be null: y2 alone never. extra: float rows added as
+// they are. w1 null: no norm output; w2 needs w1. h1/h2 have dtype out_dt.
+int dsv_scaled_add(float* x, const float* s1, const void* y1, const float* s2, const void* y2,
+                   const float* extra, const float* w1, const float* w2, void* h1, void* h2,
+                   int dt, int out_dt, int rows, int C, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if ((y1 && !s1) || (y2 && (!y1 || !s2)) || (w1 && !h1) || (w2 && (!w1 || !h2))) return -1;
+  const bool vec = C % 8 == 0 && C <= 8 * NT * LN_G;
+#define SA(T, TO)                                                                              \
+  do {                                                                                         \
+    if (vec)                                                                                   \
+      scaled_add_k<T, TO, true><<<rows, NT, 0, s>>>(x, s1, (const T*)y1, s2, (const T*)y2,     \
+                                                    extra, w1, w2, (TO*)h1, (TO*)h2, C, eps);  \
+    else                                                                                       \
+      scaled_add_k<T, TO, false><<<rows, NT, 0, s>>>(x, s1, (const T*)y1, s2, (const T*)y2,    \
+                                                     extra, w1, w2, (TO*)h1, (TO*)h2, C, eps); \
+  } while (0)
+  if (dt == 0 && out_dt == 0) SA(float, float);
+  else if (dt == 0) SA(float, bf16);
+  else if (out_dt == 0) SA(bf16, float);
+  else SA(bf16, bf16);
+#undef SA
   return (int)hipGetLastError();
 }
 

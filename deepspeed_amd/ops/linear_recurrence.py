@@ -29,8 +29,10 @@ Around the scan:
 * ``gate_group_norm``: the read-out plus the skip ``D * x``, times
   ``silu(gate)``, then an RMS norm over equal parts of the row, times a weight.
 * ``sigmoid_pow``: ``sigmoid(z + bias) ** (1 / tau)`` for per-channel decays.
+* ``softplus_decay``: ``exp(-exp(A_log_h) * softplus(z + bias))`` per head and
+  key channel (the delta rule with a decay of its own for every row of S).
 * ``head_norm_gate``: per-head RMS norm of the read-out times a weight shared
-  by the heads, times ``silu(gate)``.
+  by the heads, times ``silu(gate)`` or ``sigmoid(gate)``.
 """
 
 import torch
@@ -52,10 +54,13 @@ def unit_heads(x, scale=1.0):
 
 
 def delta_prep(proj, batch, conv_w, conv_state, a_log, dt_bias, kv_heads,
-               heads, dim, vdim):
-    """proj [T, 2*kv_heads*dim + 2*heads*vdim + 2*heads] =
-    q | k | v | gate | b | a (the gate columns are left for
-    ``head_norm_gate``). conv_w [2*kv_heads*dim + heads*vdim, taps] and
+               heads, dim, vdim, beta_col=None, a_col=None):
+    """proj [T, ...] starts with q | k | v; by default the row goes on
+    ``| gate | b | a`` (the gate columns are left for ``head_norm_gate``).
+    ``beta_col`` / ``a_col`` name the first of the ``heads`` columns of b and
+    of a in other layouts; ``a_col=-1`` makes no per-head decay here (the
+    caller has one per key channel, see ``softplus_decay``) and returns None
+    for it. conv_w [2*kv_heads*dim + heads*vdim, taps] and
     conv_state [slots, taps-1, same] cover the q|k|v columns.
     Returns fp32 q [T, kv_heads, dim] (unit length times dim^-1/2),
     k [T, kv_heads, dim] (unit length), v [T, heads, vdim], beta [T, heads],
@@ -63,18 +68,38 @@ def delta_prep(proj, batch, conv_w, conv_state, a_log, dt_bias, kv_heads,
     T = proj.shape[0]
     nqk, nv = kv_heads * dim, heads * vdim
     C = 2 * nqk + nv
-    assert proj.shape[1] == C + nv + 2 * heads and conv_w.shape[0] == C
+    if beta_col is None:
+        assert proj.shape[1] == C + nv + 2 * heads
+        beta_col = C + nv
+    if a_col is None:
+        a_col = beta_col + heads
+    assert conv_w.shape[0] == C
     if proj.is_cuda and _sk().enabled():
         return _sk().delta_prep(proj, batch, conv_w, conv_state, a_log,
-                                dt_bias, kv_heads, heads, dim, vdim)
+                                dt_bias, kv_heads, heads, dim, vdim,
+                                beta_col, a_col)
     y = conv_silu_ragged(proj[:, :C], conv_w, conv_state, batch)
     q = unit_heads(y[:, :nqk].reshape(T, kv_heads, dim), dim ** -0.5)
     k = unit_heads(y[:, nqk:2 * nqk].reshape(T, kv_heads, dim))
     v = y[:, 2 * nqk:].reshape(T, heads, vdim)
-    beta = torch.sigmoid(proj[:, C + nv:C + nv + heads].float())
-    dt = F.softplus(proj[:, C + nv + heads:].float() + dt_bias.float())
-    decay = torch.exp(-torch.exp(a_log.float()) * dt)
+    beta = torch.sigmoid(proj[:, beta_col:beta_col + heads].float())
+    decay = None
+    if a_col >= 0:
+        dt = F.softplus(proj[:, a_col:a_col + heads].float()
+                        + dt_bias.float())
+        decay = torch.exp(-torch.exp(a_log.float()) * dt)
     return q.contiguous(), k.contiguous(), v.contiguous(), beta, decay
+
+
+def softplus_decay(z, bias, a_log, heads):
+    """Per head and key channel: ``exp(-exp(a_log_h) * softplus(z + bias))``
+    in fp32. z [T, heads*dim] (a projection, may be a column slice),
+    bias [heads*dim], a_log [heads]. Returns [T, heads, dim]."""
+    if z.is_cuda and _sk().enabled():
+        return _sk().softplus_decay(z, bias, a_log, heads)
+    T, C = z.shape
+    dt = F.softplus(z.float() + bias.float()).view(T, heads, C // heads)
+    return torch.exp(-torch.exp(a_log.float())[None, :, None] * dt)
 
 
 def sigmoid_pow(z, bias, inv_tau):
@@ -120,16 +145,19 @@ def linear_scan(q, k, v, decay, beta, state, batch, q_scale=1.0):
     return out
 
 
-def head_norm_gate(o, weight, gate, eps, out_dtype):
+def head_norm_gate(o, weight, gate, eps, out_dtype, act="silu"):
     """o [T, H, vdim] fp32; weight [vdim]; gate [T, H*vdim] pre-activation
     (may be a column slice). Returns
-    ``o / sqrt(mean_v(o^2) + eps) * weight * silu(gate)`` as
-    [T, H*vdim] ``out_dtype``."""
+    ``o / sqrt(mean_v(o^2) + eps) * weight * act(gate)`` as
+    [T, H*vdim] ``out_dtype``; ``act`` is "silu" or "sigmoid"."""
     T, H, vdim = o.shape
+    if act not in ("silu", "sigmoid"):
+        raise ValueError(f"unknown gate activation {act!r}")
     if o.is_cuda and _sk().enabled():
-        return _sk().head_norm_gate(o, weight, gate, eps, out_dtype)
+        return _sk().head_norm_gate(o, weight, gate, eps, out_dtype, act)
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
-    return (y.reshape(T, H * vdim) * F.silu(gate.float())).to(out_dtype)
+    g = F.silu(gate.float()) if act == "silu" else torch.sigmoid(gate.float())
+    return (y.reshape(T, H * vdim) * g).to(out_dtype)
 
 
 def ssd_prep(proj, batch, conv_w, conv_b, conv_state, a_log, dt_bias, heads,

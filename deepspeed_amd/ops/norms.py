@@ -205,22 +205,31 @@ def layer_norm_rows(x, weight, bias, eps, out_dtype=None, index=None):
             + bias.float()).to(out_dtype)
 
 
-def embed_rows(table, ids, scale, out_dtype=torch.float32):
-    """``table[ids] * scale`` in fp32, rounded once to ``out_dtype``."""
+def embed_rows(table, ids, scale, out_dtype=torch.float32, add_table=None,
+               add_ids=None):
+    """``table[ids] * scale`` in fp32, rounded once to ``out_dtype``. With
+    ``add_table`` the rows ``add_table[add_ids]`` (a second table of the same
+    width, e.g. a hashed one) are added in fp32 in the same pass."""
     if table.is_cuda and _sk().enabled():
-        return _sk().embed_rows(table, ids, scale, out_dtype)
-    return (table[ids].float() * scale).to(out_dtype)
+        return _sk().embed_rows(table, ids, scale, out_dtype, add_table,
+                                add_ids)
+    out = table[ids].float() * scale
+    if add_table is not None:
+        out = out + add_table[add_ids].float()
+    return out.to(out_dtype)
 
 
 def rms_norm_rows(x, weight, eps, out_dtype=None, index=None, one_plus=False):
     """RMS norm with a weight per coordinate of the rows ``x[index]`` (all
     rows without ``index``): ``x / sqrt(mean(x^2) + eps) * w``, or
     ``* (1 + w)`` with ``one_plus`` (weights stored around zero). fp32
-    statistics and product, rounded once to ``out_dtype``."""
+    statistics and product, rounded once to ``out_dtype``. ``x`` may be a
+    column slice of a wider tensor."""
     out_dtype = out_dtype or x.dtype
     if x.is_cuda and _sk().enabled():
-        return _sk().rms_norm_rows(x.contiguous(), weight, eps, out_dtype,
-                                   index, one_plus)
+        if x.stride(-1) != 1:
+            x = x.contiguous()
+        return _sk().rms_norm_rows(x, weight, eps, out_dtype, index, one_plus)
     xf = (x if index is None else x[index]).float()
     w = weight.float() + 1.0 if one_plus else weight.float()
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
@@ -246,3 +255,34 @@ def gated_add_(x, g1, y1, g2=None, y2=None, norm_weight=None, eps=1e-6,
     if norm_weight is None:
         return None
     return rms_norm_rows(x, norm_weight, eps, out_dtype, None, one_plus)
+
+
+def scaled_add_(x, s1=None, y1=None, s2=None, y2=None, extra=None,
+                norm_w1=None, norm_w2=None, eps=1e-6, out_dtype=None):
+    """Residual add with a learned factor per column on an fp32 stream, in
+    place: ``x += s1 * y1 (+ s2 * y2) (+ extra)``. ``y*`` are sublayer results
+    ([T, C], any float type), ``s*`` fp32 [C], ``extra`` fp32 [T, C] added as
+    it is; products and the sum are fp32. All three may be absent (the row is
+    then only normed). With ``norm_w1`` (and ``norm_w2``) the same pass
+    returns the RMS norms ``x / sqrt(mean(x^2) + eps) * w`` of the NEW row
+    under each weight in ``out_dtype``: two sublayers that read one row
+    through norms of their own share the read and the statistic.
+    Returns (h1, h2), None where no weight was given."""
+    assert x.dtype == torch.float32
+    if x.is_cuda and _sk().enabled():
+        return _sk().scaled_add(x, s1, y1, s2, y2, extra, norm_w1, norm_w2,
+                                eps, out_dtype)
+    if y1 is not None:
+        d = s1.float() * y1.float()
+        if y2 is not None:
+            d = d + s2.float() * y2.float()
+        x.add_(d)
+    if extra is not None:
+        x.add_(extra)
+    if norm_w1 is None:
+        return None, None
+    out_dtype = out_dtype or torch.float32
+    n = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    h1 = (n * norm_w1.float()).to(out_dtype)
+    h2 = None if norm_w2 is None else (n * norm_w2.float()).to(out_dtype)
+    return h1, h2

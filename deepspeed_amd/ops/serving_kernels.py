@@ -197,30 +197,44 @@ def residual_add_stats(x, delta):
 
 
 # ------------------------------------------------------ latent attention
-def latent_prep(proj, batch, pool, norm_w, eps, heads, dim, rot, rank,
-                rot_dims, cos, sin):
-    T = proj.shape[0]
-    assert proj.is_contiguous() and proj.dtype == pool.dtype
-    assert proj.shape[1] == heads * (dim + rot) + rank + rot + heads
+def latent_prep(q, kv, gate_z, batch, pool, norm_w, eps, heads, dim, rot, rank,
+                rot_dims, cos, sin, layout="interleaved"):
+    """q [T, heads*(dim+rot)], kv [T, rank+rot], gate_z [T, heads] or None:
+    column slices (rows contiguous) of one or of several projections."""
+    T = q.shape[0]
+    for t in (q, kv) + (() if gate_z is None else (gate_z,)):
+        _rows_ok(t)
+        assert t.dtype == pool.dtype and t.shape[0] == T
+    assert q.shape[1] == heads * (dim + rot) and kv.shape[1] == rank + rot
+    assert gate_z is None or gate_z.shape[1] == heads
     assert pool.shape[-1] == rank + rot and T == batch.n_tokens
     assert rot_dims % 2 == 0 and rot_dims <= rot
-    assert cos.shape[1] == rot_dims // 2 and cos.shape[0] >= batch.max_ctx
-    assert cos.dtype == torch.float32 and sin.shape == cos.shape
-    dev, dt = proj.device, proj.dtype
+    assert layout in ("interleaved", "half")
+    if rot_dims:
+        assert cos.shape[1] == rot_dims // 2 and cos.shape[0] >= batch.max_ctx
+        assert cos.dtype == torch.float32 and sin.shape == cos.shape
+    dev, dt = q.device, q.dtype
     q_nope = torch.empty(heads, T, dim, dtype=dt, device=dev)
-    q_rot = torch.empty(T, heads, rot, dtype=dt, device=dev)
-    gate = torch.empty(T, heads, dtype=torch.float32, device=dev)
+    q_rot = torch.empty(T, heads, rot, dtype=dt, device=dev) if rot else None
+    gate = None if gate_z is None else \
+        torch.empty(T, heads, dtype=torch.float32, device=dev)
     _check(load("latent").dsv_latent_prep(
-        _p(proj), _i(proj.shape[1]), _p(_f32(norm_w)), _p(batch.tok_pos),
-        _p(batch.tok_row), _p(cos), _p(sin), _p(pool), _p(q_nope), _p(q_rot),
-        _p(gate), _i(_dt(proj)), _i(T), _i(heads), _i(dim), _i(rot), _i(rank),
-        _i(rot_dims), _f(eps), _stream()), "latent_prep")
+        _vp(q), _i(q.stride(0)), _vp(kv), _i(kv.stride(0)),
+        _p(None) if gate_z is None else _vp(gate_z),
+        _i(0 if gate_z is None else gate_z.stride(0)), _p(_f32(norm_w)),
+        _p(batch.tok_pos), _p(batch.tok_row), _p(cos if rot_dims else None),
+        _p(sin if rot_dims else None), _p(pool), _p(q_nope), _p(q_rot),
+        _p(gate), _i(_dt(q)), _i(T), _i(heads), _i(dim), _i(rot), _i(rank),
+        _i(rot_dims), _f(eps), _i(1 if layout == "half" else 0), _stream()),
+        "latent_prep")
     return q_nope, q_rot, gate
 
 
-def _attn_plan(batch, dtype, rank, rot):
+def _attn_plan(batch, dtype, rank, rot, reach=None):
     """Key-chunk length that fits LDS, and the number of key splits: few
-    tokens over a long history are split so the launch still fills the chip."""
+    tokens over a long history are split so the launch still fills the chip.
+    ``reach``: the most keys a token sees (a window bounds it)."""
+    reach = batch.max_ctx if reach is None else reach
     lib = load("latent")
     dt = _DT[dtype]
     kc = 64
@@ -228,7 +242,7 @@ def _attn_plan(batch, dtype, rank, rot):
         kc //= 2
     nsplit = 1
     if batch.n_tokens <= 128:
-        nsplit = max(1, min(32, batch.max_ctx // (4 * kc),
+        nsplit = max(1, min(32, reach // (4 * kc),
                             1024 // max(1, batch.n_tokens)))
     return kc, nsplit
 
@@ -249,17 +263,25 @@ def _tile_work(batch, heads, tile_rows, device):
     return batch.extra[key]
 
 
-def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None):
-    """``path`` forces "mfma" or "exact" (tests); default chooses by size."""
+def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None,
+                     window=0, sink=None):
+    """``path`` forces "mfma" or "exact" (tests); default chooses by size.
+    ``q_rot`` is None when rows hold no rotated part."""
     H, T, r = q_lat.shape
-    rot = q_rot.shape[2]
-    assert r == rank and q_rot.shape[:2] == (T, H) and T == batch.n_tokens
+    rot = 0 if q_rot is None else q_rot.shape[2]
+    assert r == rank and T == batch.n_tokens and window >= 0
     assert pool.shape[-1] == rank + rot and pool.shape[1] == batch.block_size
-    assert q_lat.dtype == pool.dtype == q_rot.dtype
-    assert q_rot.is_contiguous() and pool.is_contiguous()
+    assert q_lat.dtype == pool.dtype and pool.is_contiguous()
+    if rot:
+        assert q_rot.shape[:2] == (T, H) and q_rot.dtype == pool.dtype
+        assert q_rot.is_contiguous()
+    if sink is not None:
+        assert sink.numel() == H
+        sink = _f32(sink).contiguous()
     q_lat = q_lat.contiguous()
     lib = load("latent")
     out = torch.empty_like(q_lat)
+    reach = min(batch.max_ctx, window) if window > 0 else batch.max_ctx
     mfma = q_lat.dtype == torch.bfloat16 and \
         lib.dsv_latent_attn_mfma_ok(_i(rank), _i(rot)) == 1
     if path is None:
@@ -272,7 +294,7 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None):
         # launch still covers the chip; partial sums are merged in fp32
         nsplit = 1
         if n < 128:
-            nsplit = max(1, min(32, batch.max_ctx // 128, 512 // n))
+            nsplit = max(1, min(32, reach // 128, 512 // n))
         part = None
         if nsplit > 1:
             part = torch.empty(T, nsplit, H, rank + 2, dtype=torch.float32,
@@ -282,9 +304,9 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None):
             _p(batch.seq_start), _p(batch.block_table),
             _i(batch.block_table.shape[1]), _i(batch.block_size), _p(out),
             _p(part), _i(T), _i(H), _i(rank), _i(rot), _i(nsplit), _f(scale),
-            _stream()), "latent_attention(mfma)")
+            _i(window), _p(sink), _stream()), "latent_attention(mfma)")
         return out
-    kc, nsplit = _attn_plan(batch, q_lat.dtype, rank, rot)
+    kc, nsplit = _attn_plan(batch, q_lat.dtype, rank, rot, reach)
     part = None
     if nsplit > 1:
         part = torch.empty(T, nsplit, H, rank + 2, dtype=torch.float32,
@@ -293,14 +315,15 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None):
         _p(q_lat), _p(q_rot), _p(pool), _p(batch.tok_seq), _p(batch.tok_pos),
         _p(batch.block_table), _i(batch.block_table.shape[1]),
         _i(batch.block_size), _p(out), _p(part), _i(_dt(q_lat)), _i(T), _i(H),
-        _i(rank), _i(rot), _i(kc), _i(nsplit), _f(scale), _stream()),
-        "latent_attention")
+        _i(rank), _i(rot), _i(kc), _i(nsplit), _f(scale), _i(window),
+        _p(sink), _stream()), "latent_attention")
     return out
 
 
-def gate_merge_heads(o, gate):
+def gate_merge_heads(o, gate=None):
     H, T, v = o.shape
-    assert gate.shape == (T, H) and gate.dtype == torch.float32
+    assert gate is None or (gate.shape == (T, H)
+                            and gate.dtype == torch.float32)
     out = torch.empty(T, H * v, dtype=o.dtype, device=o.device)
     _check(load("latent").dsv_gate_merge(_p(o.contiguous()), _p(gate), _p(out),
                                  _i(_dt(o)), _i(T), _i(H), _i(v), _stream()),
@@ -388,15 +411,35 @@ def layer_norm_rows(x, weight, bias, eps, out_dtype, index=None):
     return out
 
 
-def embed_rows(table, ids, scale, out_dtype=torch.float32):
+def embed_rows(table, ids, scale, out_dtype=torch.float32, add_table=None,
+               add_ids=None):
     assert table.is_contiguous() and table.dim() == 2
     ids = ids.to(torch.int64).contiguous()
+    if add_table is not None:
+        assert add_table.is_contiguous() and add_table.dtype == table.dtype
+        assert add_table.shape[1] == table.shape[1]
+        add_ids = add_ids.to(torch.int64).contiguous()
+        assert add_ids.numel() == ids.numel()
     out = torch.empty(ids.numel(), table.shape[1], dtype=torch.float32,
                       device=table.device)
-    _check(load().dsv_embed_rows(_p(table), _i(_dt(table)), _p(ids), _p(out),
+    _check(load().dsv_embed_rows(_p(table), _i(_dt(table)), _p(ids),
+                                 _p(add_table), _p(add_ids), _p(out),
                                  _i(ids.numel()), _i(table.shape[1]),
                                  _f(scale), _stream()), "embed_rows")
     return out if out_dtype == torch.float32 else out.to(out_dtype)
+
+
+def pair_hash_rows(ids, batch, prev, mul_prev, mul_cur, buckets):
+    T = ids.numel()
+    assert T == batch.n_tokens and ids.dtype == torch.int64
+    assert prev.dtype == torch.int64 and prev.dim() == 1
+    ids = ids.contiguous()
+    rows = torch.empty(T, dtype=torch.int64, device=ids.device)
+    _check(load().dsv_pair_hash_rows(
+        _p(ids), _p(batch.cu), _p(batch.seq_slot), _p(batch.tok_seq),
+        _p(batch.tok_pos), _p(prev), _p(rows), _i(T), _i(batch.n_seqs),
+        _l(mul_prev), _l(mul_cur), _l(buckets), _stream()), "pair_hash_rows")
+    return rows
 
 
 def glu(gu, act):
@@ -410,14 +453,22 @@ def glu(gu, act):
 
 
 def grouped_sigmoid_topk(logits, correction, top, groups, keep):
+    return grouped_topk(logits, correction, top, groups, keep, "sigmoid",
+                        "top2", False, 1.0)
+
+
+def grouped_topk(logits, correction, top, groups, keep, score, group_score,
+                 renorm, scale):
     T, E = logits.shape
     assert logits.dtype == torch.float32 and correction.numel() == E
     idx = torch.empty(T, top, dtype=torch.int64, device=logits.device)
     w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    _check(load().dsv_grouped_sigmoid_topk(
+    _check(load().dsv_grouped_topk(
         _p(logits.contiguous()), _p(_f32(correction).contiguous()), _p(idx),
-        _p(w), _i(T), _i(E), _i(top), _i(groups), _i(keep), _stream()),
-        "grouped_sigmoid_topk")
+        _p(w), _i(T), _i(E), _i(top), _i(groups), _i(keep),
+        _i(("sigmoid", "softmax").index(score)),
+        _i(("top2", "max").index(group_score)), _i(1 if renorm else 0),
+        _f(scale), _stream()), "grouped_topk")
     return idx, w
 
 
@@ -584,10 +635,16 @@ def window_attention(q, pool, batch, kv_heads, dim, vdim, scale, window=0,
 
 # ------------------------------------------------------ linear recurrences
 def delta_prep(proj, batch, conv_w, conv_state, a_log, dt_bias, kv_heads,
-               heads, dim, vdim):
+               heads, dim, vdim, beta_col=None, a_col=None):
     T = proj.shape[0]
     taps = conv_w.shape[1]
     C = 2 * kv_heads * dim + heads * vdim
+    if beta_col is None:
+        beta_col = C + heads * vdim
+    if a_col is None:
+        a_col = beta_col + heads
+    assert 0 <= beta_col <= proj.shape[1] - heads
+    assert a_col < 0 or a_col <= proj.shape[1] - heads
     assert proj.is_contiguous() and T == batch.n_tokens
     assert conv_w.dtype == proj.dtype == conv_state.dtype
     assert conv_w.is_contiguous() and conv_w.shape[0] == C
@@ -600,16 +657,32 @@ def delta_prep(proj, batch, conv_w, conv_state, a_log, dt_bias, kv_heads,
     k = torch.empty(T, kv_heads, dim, **f32)
     v = torch.empty(T, heads, vdim, **f32)
     beta = torch.empty(T, heads, **f32)
-    decay = torch.empty(T, heads, **f32)
+    decay = torch.empty(T, heads, **f32) if a_col >= 0 else None
     _check(_seq().dsv_delta_prep(
         _p(proj), _i(proj.shape[1]), _p(conv_w),
         ctypes.c_void_p(conv_state.data_ptr()), _l(conv_state.stride(0)),
         _p(batch.cu), _p(batch.seq_slot), _p(batch.seq_start),
-        _p(batch.tok_seq), _p(batch.tok_pos), _p(_f32(a_log)),
-        _p(_f32(dt_bias)), _p(q), _p(k), _p(v), _p(beta), _p(decay),
+        _p(batch.tok_seq), _p(batch.tok_pos),
+        _p(_f32(a_log) if a_col >= 0 else None),
+        _p(_f32(dt_bias) if a_col >= 0 else None), _p(q), _p(k), _p(v),
+        _p(beta), _p(decay),
         _i(_dt(proj)), _i(T), _i(batch.n_seqs), _i(kv_heads), _i(heads),
-        _i(dim), _i(vdim), _i(taps), _stream()), "delta_prep")
+        _i(dim), _i(vdim), _i(taps), _i(beta_col), _i(a_col), _stream()),
+        "delta_prep")
     return q, k, v, beta, decay
+
+
+def softplus_decay(z, bias, a_log, heads):
+    T, C = z.shape
+    _rows_ok(z)
+    assert C % heads == 0 and bias.numel() == C and a_log.numel() == heads
+    out = torch.empty(T, heads, C // heads, dtype=torch.float32,
+                      device=z.device)
+    _check(_seq().dsv_softplus_decay(
+        _vp(z), _i(z.stride(0)), _p(_f32(bias).contiguous()),
+        _p(_f32(a_log).contiguous()), _p(out), _i(_dt(z)), _l(T), _i(heads),
+        _i(C // heads), _stream()), "softplus_decay")
+    return out
 
 
 def sigmoid_pow(z, bias, inv_tau):
@@ -652,7 +725,7 @@ def linear_scan(q, k, v, decay, beta, state, batch, q_scale=1.0):
     return out
 
 
-def head_norm_gate(o, weight, gate, eps, out_dtype):
+def head_norm_gate(o, weight, gate, eps, out_dtype, act="silu"):
     T, H, vdim = o.shape
     assert o.dtype == torch.float32 and o.is_contiguous()
     assert weight.numel() == vdim and gate.shape == (T, H * vdim)
@@ -662,7 +735,8 @@ def head_norm_gate(o, weight, gate, eps, out_dtype):
     _check(_seq().dsv_head_norm_gate(
         _p(o), _p(_f32(weight)), ctypes.c_void_p(gate.data_ptr()),
         _i(gate.stride(0)), _p(out), _i(_DT[out_dtype]), _i(T), _i(H),
-        _i(vdim), _f(eps), _stream()), "head_norm_gate")
+        _i(vdim), _f(eps), _i(("silu", "sigmoid").index(act)), _stream()),
+        "head_norm_gate")
     return out
 
 
@@ -765,15 +839,50 @@ def selective_scan(x, dt_pre, dt_bias, a_log, B, C, skip, z, state, batch,
 def rms_norm_rows(x, weight, eps, out_dtype, index=None, one_plus=False):
     rows = x.shape[0] if index is None else index.numel()
     C = x.shape[1]
-    assert weight.numel() == C and x.is_contiguous()
+    _rows_ok(x)
+    assert weight.numel() == C
     out = torch.empty(rows, C, dtype=out_dtype, device=x.device)
     if index is not None:
         index = index.to(torch.int64).contiguous()
     _check(load().dsv_rms_norm_rows(
-        _p(x), _i(_dt(x)), _p(index), _p(_f32(weight)), _p(out),
-        _i(_DT[out_dtype]), _i(rows), _i(C), _f(eps), _i(1 if one_plus else 0),
-        _stream()), "rms_norm_rows")
+        _vp(x), _i(_dt(x)), _i(x.stride(0)), _p(index), _p(_f32(weight)),
+        _p(out), _i(_DT[out_dtype]), _i(rows), _i(C), _f(eps),
+        _i(1 if one_plus else 0), _stream()), "rms_norm_rows")
     return out
+
+
+def scaled_add(x, s1, y1, s2, y2, extra, w1, w2, eps, out_dtype):
+    """x += s1*y1 (+ s2*y2) (+ extra) in place; returns (h1, h2): the RMS
+    norms of the new x under w1 / w2 (None where no weight is given)."""
+    T, C = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    dt = _dt(x)
+    if y1 is not None:
+        y1 = y1.contiguous()
+        assert y1.shape == (T, C) and s1.numel() == C
+        dt = _dt(y1)
+    if y2 is not None:
+        y2 = y2.contiguous()
+        assert y1 is not None and y2.shape == (T, C) and s2.numel() == C
+        assert y2.dtype == y1.dtype
+    if extra is not None:
+        assert extra.shape == (T, C) and extra.dtype == torch.float32
+        extra = extra.contiguous()
+    h1 = h2 = None
+    out_dtype = out_dtype or torch.float32
+    if w1 is not None:
+        assert w1.numel() == C
+        h1 = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    if w2 is not None:
+        assert w1 is not None and w2.numel() == C
+        h2 = torch.empty(T, C, dtype=out_dtype, device=x.device)
+    f = lambda t: None if t is None else _f32(t).contiguous()
+    _check(load().dsv_scaled_add(
+        _p(x), _p(f(s1) if y1 is not None else None), _p(y1),
+        _p(f(s2) if y2 is not None else None), _p(y2), _p(extra), _p(f(w1)),
+        _p(f(w2)), _p(h1), _p(h2), _i(dt), _i(_DT[out_dtype]), _i(T), _i(C),
+        _f(eps), _stream()), "scaled_add")
+    return h1, h2
 
 
 def gated_add(x, g1, y1, g2, y2, norm_weight, eps, out_dtype, one_plus):
