@@ -34,7 +34,7 @@ def parse_args():
                    help="ZeRO-Offload optimizer states to host DRAM")
     p.add_argument("--activation-checkpointing", action="store_true")
     p.add_argument("--local_rank", type=int, default=-1)
-    p.add_argument("--serving", type=str, default=None, choices=["fizesun", "lolulorn", "savovik"],
+    p.add_argument("--serving", type=str, default=None, choices=["fizesun", "lolulorn", "savovik", "numolorn"],
                    help="instead of the training step: serving throughput "
                         "(prefill, decode) of this design beside Llama at "
                         "equal size, with per-kernel roofline distances")
