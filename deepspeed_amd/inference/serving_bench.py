@@ -1011,7 +1011,7 @@ def _numolorn_kernel_rows(z, dev):
     rc = PagedStateCache([], {"conv": (3, C)}, B, B * (S + 64), dtype=bf,
                          device=dev)
     bt = rc.begin_ragged(list(range(B)), [S] * B)
-    pj = torch.randn(T, C + RH + 128, device=dev).to(bf)
+    pj = torch.randn(T, (C + RH + 128 + 7) // 8 * 8, device=dev).to(bf)
     pl = torch.randn(T, C + RH * rv + 2 * RH, device=dev).to(bf)
     cw = torch.randn(C, 4, device=dev).to(bf)
     al, db = torch.zeros(RH, device=dev), torch.zeros(RH, device=dev)

@@ -540,8 +540,12 @@ class NumolornForCausalLM(nn.Module):
                 taps.append(x.clone())
         if pending is not None:
             scaled_add_(x, *pending)
-        hn = rms_norm_rows(x, self.final_norm, eps, dt, rows)
-        return F.linear(hn, self.embed).float() * self.cfg.logit_scale
+        # logits = table . (norm(x) * w) * scale: the scale rides on the
+        # norm's weight, so no pass over [rows, vocab] is needed for it
+        w = self.final_norm
+        if self.cfg.logit_scale != 1.0:
+            w = w * self.cfg.logit_scale
+        return F.linear(rms_norm_rows(x, w, eps, dt, rows), self.embed)
 
     def num_parameters(self):
         return sum(p.numel() for p in self.parameters())

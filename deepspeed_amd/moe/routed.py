@@ -208,15 +208,12 @@ class RoutedExperts(nn.Module):
                                       self.w_gu.transpose(1, 2)))
             y = torch.bmm(mid, self.w_down.transpose(1, 2)) \
                 .reshape(self.experts * T, -1)
-            inv = idx * T + torch.arange(T, device=h.device)[:, None]
             if self.identity:
                 # identity outputs all read the token's own row, kept once
-                # after the experts' results
+                # after the experts' results: block number ``experts``
                 y = torch.cat([y, h], 0)
-                inv = torch.where(idx >= self.experts,
-                                  self.experts * T
-                                  + torch.arange(T, device=h.device)[:, None],
-                                  inv)
+                idx = idx.clamp(max=self.experts)
+            inv = idx * T + torch.arange(T, device=h.device)[:, None]
         else:
             y, inv = self._grouped(h, idx)
         sh = sg = None

@@ -470,6 +470,28 @@ __global__ void clamped_swiglu_k(const T* __restrict__ gu, T* __restrict__ out,
   }
 }
 
+// the same, eight columns per thread (F a multiple of 8)
+template <typename T>
+__global__ void clamped_swiglu8_k(const T* __restrict__ gu, T* __restrict__ out, int64_t rows,
+                                  int F, float limit) {
+  const int F8 = F >> 3;
+  const int64_t n = rows * F8;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / F8;
+    const int c = (int)(i - r * F8) << 3;
+    float g[8], u[8];
+    load8(gu + r * 2 * F + c, g);
+    load8(gu + r * 2 * F + F + c, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gc = fminf(g[e], limit);
+      const float uc = fminf(fmaxf(u[e], -limit), limit);
+      g[e] = gc / (1.f + expf(-1.702f * gc)) * (uc + 1.f);
+    }
+    store8(out + r * F + c, g);
+  }
+}
 
 // gu [rows, 2F] (gate | up) -> act(gate) * up; ACT 0 = silu, 1 = tanh-form gelu
 template <typename T, int ACT>
@@ -570,13 +592,19 @@ __global__ void grouped_topk_k(const float* __restrict__ z, const float* __restr
     }
   }
   float total = 0.f;
+  // experts already chosen: a bit each in a register while they fit, else
+  // read back from the output row
+  unsigned long long chosen = 0ull;
   for (int k = 0; k < top; ++k) {
     int bi = -1;
     float bv = -INFINITY, bs = 0.f;
     for (int e = 0; e < E; ++e) {
       if (!((allowed >> (e / per)) & 1ull)) continue;
       bool taken = false;
-      for (int q = 0; q < k; ++q) taken |= idx[(int64_t)t * top + q] == e;
+      if (E <= 64)
+        taken = (chosen >> e) & 1ull;
+      else
+        for (int q = 0; q < k; ++q) taken |= idx[(int64_t)t * top + q] == e;
       if (taken) continue;
       const float sg = score(e);
       const float c = sg + corr[e];
@@ -589,6 +617,7 @@ __global__ void grouped_topk_k(const float* __restrict__ z, const float* __restr
     idx[(int64_t)t * top + k] = bi;
     w[(int64_t)t * top + k] = bs;
     total += bs;
+    if (E <= 64 && bi >= 0) chosen |= 1ull << bi;
   }
   const float f = renorm ? scale / (total + 1e-20f) : scale;
   if (renorm || scale != 1.f)
@@ -1068,6 +1097,11 @@ int dsv_xielu(const void* z, const float* pq, void* out, int dt, int64_t n, hipS
 int dsv_clamped_swiglu(const void* gu, void* out, int dt, int64_t rows, int F, float limit,
                        hipStream_t s) {
   if (rows * F <= 0) return 0;
+  if (F % 8 == 0) {
+    BY_DTYPE(dt, (clamped_swiglu8_k<T><<<nblocks(rows * (F / 8), 256), 256, 0, s>>>(
+                     (const T*)gu, (T*)out, rows, F, limit)));
+    return (int)hipGetLastError();
+  }
   BY_DTYPE(dt, (clamped_swiglu_k<T><<<nblocks(rows * F, 256), 256, 0, s>>>((const T*)gu, (T*)out, rows, F, limit)));
   return (int)hipGetLastError();
 }
