@@ -264,8 +264,9 @@ def _tile_work(batch, heads, tile_rows, device):
 
 
 def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None,
-                     window=0, sink=None):
-    """``path`` forces "mfma" or "exact" (tests); default chooses by size.
+                     window=0, sink=None, splits=None):
+    """``path`` forces "mfma" or "exact" and ``splits`` the number of key
+    splits of the tile kernel (tests, tuning); default chooses by size.
     ``q_rot`` is None when rows hold no rotated part."""
     H, T, r = q_lat.shape
     rot = 0 if q_rot is None else q_rot.shape[2]
@@ -291,10 +292,15 @@ def latent_attention(q_lat, q_rot, pool, batch, rank, scale, path=None,
         rows = lib.dsv_latent_attn_mfma_rows(_i(rank), _i(rot))
         work, n = _tile_work(batch, H, rows, q_lat.device)
         # few tiles over long histories (decoding): split the keys so the
-        # launch still covers the chip; partial sums are merged in fp32
+        # launch still covers the chip (about one workgroup per CU: every
+        # further split writes and re-reads fp32 partial sums of rank + 2
+        # numbers per head, which at 64 requests costs more than the shorter
+        # key walk saves); partial sums are merged in fp32
         nsplit = 1
         if n < 128:
-            nsplit = max(1, min(32, reach // 128, 512 // n))
+            nsplit = max(1, min(32, reach // 128, 256 // n))
+        if splits is not None:
+            nsplit = max(1, min(int(splits), 64))
         part = None
         if nsplit > 1:
             part = torch.empty(T, nsplit, H, rank + 2, dtype=torch.float32,
