@@ -818,8 +818,8 @@ def numolorn_config(z, vocab=32000):
                "mlp": kinds[i % 4][2]} for i in range(z["layers"])]
     return {"architecture": "Numolorn", "vocab": vocab, "width": z["width"],
             "norm": {"eps": 1e-6}, "logit_scale": 1.0,
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31,
-                                     "mul_cur": 17}},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1009,
+                                     "mul_cur": 7}},
             "layers": layers}
 
 

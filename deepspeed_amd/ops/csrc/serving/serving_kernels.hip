@@ -624,18 +624,22 @@ __global__ void grouped_topk_k(const float* __restrict__ z, const float* __restr
     for (int k = 0; k < top; ++k) w[(int64_t)t * top + k] *= f;
 }
 
-// out[t] = sum_k w[t,k] * y[inv[t,k]] (+ sigmoid(sg[t]) * shared[t])
+// out[t] = sum_k w[t,k] * y[inv[t,k]] (+ sigmoid(sg[t]) * shared[t]); several
+// picks may name one row of y (identity outputs), a row index outside y's
+// nrows rows is skipped rather than read
 template <typename T>
 __global__ void moe_combine_k(const T* __restrict__ y, const int64_t* __restrict__ inv,
                               const float* __restrict__ w, const T* __restrict__ shared,
                               const T* __restrict__ sg, T* __restrict__ out,
-                              int top, int C) {
+                              int top, int C, int64_t nrows) {
   const int64_t t = blockIdx.x;
   const float g = shared ? 1.f / (1.f + expf(-ld(sg + t))) : 0.f;
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float a = 0.f;
-    for (int k = 0; k < top; ++k)
-      a += w[t * top + k] * ld(y + inv[t * top + k] * C + c);
+    for (int k = 0; k < top; ++k) {
+      const int64_t r = inv[t * top + k];
+      if (r >= 0 && r < nrows) a += w[t * top + k] * ld(y + r * C + c);
+    }
     if (shared) a += g * ld(shared + t * C + c);
     st(out + t * C + c, a);
   }
@@ -1106,11 +1110,12 @@ int dsv_clamped_swiglu(const void* gu, void* out, int dt, int64_t rows, int F, f
   return (int)hipGetLastError();
 }
 
-int dsv_moe_combine(const void* y, const int64_t* inv, const float* w, const void* shared,
-                    const void* sg, void* out, int dt, int Ttok, int top, int C, hipStream_t s) {
+int dsv_moe_combine(const void* y, int64_t nrows, const int64_t* inv, const float* w,
+                    const void* shared, const void* sg, void* out, int dt, int Ttok, int top,
+                    int C, hipStream_t s) {
   if (Ttok <= 0) return 0;
   BY_DTYPE(dt, (moe_combine_k<T><<<Ttok, 256, 0, s>>>((const T*)y, inv, w, (const T*)shared,
-                                                     (const T*)sg, (T*)out, top, C)));
+                                                     (const T*)sg, (T*)out, top, C, nrows)));
   return (int)hipGetLastError();
 }
 

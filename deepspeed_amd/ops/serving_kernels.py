@@ -360,14 +360,14 @@ def clamped_swiglu(gu, limit):
 def moe_combine(y, inv, weight, shared=None, shared_gate=None):
     T, top = inv.shape
     C = y.shape[1]
-    assert y.shape[0] >= T * top and weight.shape == (T, top)
+    assert y.dim() == 2 and y.is_contiguous() and weight.shape == (T, top)
     assert inv.dtype == torch.int64 and weight.dtype == torch.float32
     if shared is not None:
         assert shared.shape == (T, C) and shared_gate.numel() == T
         assert shared.dtype == y.dtype == shared_gate.dtype
     out = torch.empty(T, C, dtype=y.dtype, device=y.device)
     _check(load().dsv_moe_combine(
-        _p(y), _p(inv.contiguous()), _p(weight.contiguous()),
+        _p(y), _l(y.shape[0]), _p(inv.contiguous()), _p(weight.contiguous()),
         _p(None if shared is None else shared.contiguous()),
         _p(None if shared is None else shared_gate.contiguous()), _p(out),
         _i(_dt(y)), _i(T), _i(top), _i(C), _stream()), "moe_combine")

@@ -601,6 +601,32 @@ def test_grouped_softmax_router_against_the_oracle(n, ident, top, count,
     _same_picks(idx, wt, want)
 
 
+def _routed_against_oracle(T, experts, identity, top, count, keep):
+    cfg = config([(lw(), moe(experts=experts, top=top, identity=identity,
+                             count=count, keep=keep, limit=0.8))])
+    t = tensors(cfg, 9)
+    w = {k: v.double() for k, v in t.items()}
+    model = build_model(strip(cfg), torch.float32, t).load_named_tensors(t) \
+        .to(DEV).eval()
+    h = torch.randn(T, 24, generator=torch.Generator().manual_seed(T))
+    want = O.moe_ff(h.double(), w, "l0.mlp.", cfg["layers"][0]["mlp"])
+    close(model.layers[0].mlp(h.to(DEV)).double().cpu(), want)
+
+
+@pytest.mark.parametrize("T", [3, 70])     # both expert paths
+def test_more_picks_than_experts_when_most_outputs_are_identity(T):
+    """One expert and three identity outputs, three picks: the picks of a
+    token outnumber the rows the experts produce for it."""
+    _routed_against_oracle(T, experts=1, identity=3, top=3, count=2, keep=2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T", [3, 70])
+def test_identity_picks_on_the_combine_kernel(T):
+    _routed_against_oracle(T, experts=1, identity=3, top=3, count=2, keep=2)
+    _routed_against_oracle(T, experts=4, identity=2, top=3, count=3, keep=2)
+
+
 @pytest.mark.parametrize("T", [3, 70])     # both expert paths
 def test_routed_experts_with_identity_outputs_match_oracle(T):
     cfg = config([(lw(), moe(experts=4, top=3, identity=2, count=3, keep=2,
@@ -1064,7 +1090,7 @@ def test_tile_and_exact_attention_kernels_on_crafted_windows(
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,rank,rot,window,sink", [
-    (4, 64, 0, 40, False), (4, 128, 32, 0, True), (8, 96, 0, 130, False),
+    (4, 64, 0, 40, False), (5, 128, 32, 0, True), (8, 80, 0, 130, False),
     (3, 40, 8, 0, True), (16, 256, 64, 0, True), (2, 512, 0, 17, True)])
 def test_latent_attention_kernels_against_eager(dtype, H, rank, rot, window,
                                                 sink, monkeypatch):
@@ -1096,7 +1122,7 @@ def test_latent_attention_kernels_against_eager(dtype, H, rank, rot, window,
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,dv,taps", [
-    (6, 6, 64, 32, 4), (4, 2, 128, 64, 4), (3, 1, 20, 12, 3),
+    (6, 3, 64, 48, 4), (4, 2, 128, 64, 4), (3, 1, 20, 12, 3),
     (8, 8, 32, 128, 2), (2, 2, 256, 16, 1)])
 def test_channel_delta_kernels_against_eager(dtype, H, G, d, dv, taps,
                                              monkeypatch):
@@ -1189,7 +1215,7 @@ def test_clamped_gate_kernel_against_eager(F, dtype, monkeypatch):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("E,top,count,keep,score,group", [
-    (18, 4, 3, 2, "softmax", "max"), (10, 2, 5, 3, "softmax", "max"),
+    (20, 4, 5, 2, "softmax", "max"), (10, 2, 5, 3, "softmax", "max"),
     (8, 2, 4, 2, "sigmoid", "top2"), (64, 8, 8, 4, "softmax", "top2"),
     (7, 7, 1, 1, "softmax", "max")])
 def test_router_and_pair_hash_kernels_against_eager(E, top, count, keep,
@@ -1216,7 +1242,7 @@ def test_router_and_pair_hash_kernels_against_eager(E, top, count, keep,
         cache.lens[1] = 70
         cache.states["prev"][1] = 123
         b = cache.begin_ragged([0, 1, 2], [200, 1, 99])
-        rows = pair_hash_rows(ids, b, cache.states["prev"], 31, 17, 65521)
+        rows = pair_hash_rows(ids, b, cache.states["prev"], 1009, 7, 65521)
         cache.end_step()
         res.append((idx.gather(-1, order), w.gather(-1, order), rows,
                     cache.states["prev"].clone()))
