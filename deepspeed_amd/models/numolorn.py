@@ -291,7 +291,14 @@ class NumolornLayer(nn.Module):
         h1, h2 = scaled_add_(x, p[0], p[1], p[2], p[3], extra, self.norm1,
                              self.norm2, eps, dtype)
         y1 = self.mixer(h1, cache, stream, states)
-        y2 = self.mlp(h2) if self.mlp is not None else None
+        y2 = None
+        if isinstance(self.mlp, RoutedExperts) and h2.dtype != torch.float32:
+            # the router reads the normed row in fp32, not its 16-bit
+            # rounding: a close call is then decided as in 32-bit serving
+            y2 = self.mlp(h2, router_input=rms_norm_rows(
+                x, self.norm2, eps, torch.float32))
+        elif self.mlp is not None:
+            y2 = self.mlp(h2)
         return (self.ls1, y1, self.ls2, y2)
 
 

@@ -196,9 +196,12 @@ class RoutedExperts(nn.Module):
         return grouped_sigmoid_topk(logits, self.router_bias, self.top,
                                     *self.groups)
 
-    def forward(self, h):
+    def forward(self, h, router_input=None):
+        """``router_input``: the rows the router reads when they are at hand
+        in a wider type than ``h`` (the fp32 normed row beside its 16-bit
+        rounding); the experts read ``h``."""
         T = h.shape[0]
-        idx, weight = self.route(h)
+        idx, weight = self.route(h if router_input is None else router_input)
         picks = T * self.top
         if picks <= self.DENSE_MAX_PICKS and 2 * picks >= self.experts:
             # decode-sized steps: run every expert on every token as three
