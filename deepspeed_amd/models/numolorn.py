@@ -225,7 +225,7 @@ class ChannelDeltaRule(nn.Module):
         self.norm = _w(self.vdim, dtype=torch.float32)
         self.w_o = _w(width, nv, dtype=dtype)
 
-    row_dim = 0
+    row_dim = 0          # nothing cached per token: the state is per slot
 
     def state_shapes(self, dtype):
         return {"conv": ((max(self.taps - 1, 0), self.conv_channels), dtype),
