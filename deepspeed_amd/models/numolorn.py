@@ -94,9 +94,9 @@ class NumolornConfig:
                 raise ValueError(f"layer {i}: unknown mixer {spec['type']!r}")
         if self.loop:
             a, b, t = (int(self.loop[k]) for k in ("start", "stop", "times"))
-            if not (0 <= a < b <= len(self.layers)) or t < 1:
-                raise ValueError("loop: need 0 <= start < stop <= layers "
-                                 "and times >= 1")
+            if not (0 <= a <= b <= len(self.layers)) or t < 0:
+                raise ValueError("loop: need 0 <= start <= stop <= layers "
+                                 "and times >= 0")
         if self.bigram and int(self.bigram["buckets"]) < 1:
             raise ValueError("bigram: buckets must be positive")
 
