@@ -891,6 +891,28 @@ __global__ void softplus_decay_k(const T* __restrict__ z, int ld_z, const float*
   }
 }
 
+// the same, eight neighbouring channels per thread (dim and ld_z multiples of
+// 8, z aligned for load8): a group of 8 lies inside one head
+template <typename T>
+__global__ void softplus_decay8_k(const T* __restrict__ z, int ld_z,
+                                  const float* __restrict__ bias, const float* __restrict__ a_log,
+                                  float* __restrict__ out, int64_t rows, int H, int dim) {
+  const int C8 = (H * dim) >> 3;
+  const int64_t n = rows * C8;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / C8;
+    const int c = (int)(i - r * C8) << 3;
+    float v[8], b[8];
+    load8(z + r * ld_z + c, v);
+    load8(bias + c, b);
+    const float rate = -expf(a_log[c / dim]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = expf(rate * softplusf_(v[e] + b[e]));
+    store8(out + r * (int64_t)(C8 << 3) + c, v);
+  }
+}
+
 // ------------------------------------------------------ linear recurrence
 // S [dim, vdim] per (slot, head), float. The columns of S are independent in
 // both forms, so the work is split by column: SCAN_R lanes share a column,
@@ -1887,6 +1909,12 @@ int dsv_head_norm_gate(const float* o, const float* w, const void* gate, int ld_
 int dsv_softplus_decay(const void* z, int ld_z, const float* bias, const float* a_log, float* out,
                        int dt, int64_t rows, int H, int dim, hipStream_t s) {
   if (rows * H * dim <= 0) return 0;
+  const size_t align = dt == 0 ? 32 : 16;
+  if (dim % 8 == 0 && ld_z % 8 == 0 && (uintptr_t)z % align == 0 && (uintptr_t)bias % 32 == 0) {
+    BY_DTYPE(dt, (softplus_decay8_k<T><<<nblocks(rows * (H * dim / 8), 256), 256, 0, s>>>(
+                     (const T*)z, ld_z, bias, a_log, out, rows, H, dim)));
+    return (int)hipGetLastError();
+  }
   BY_DTYPE(dt, (softplus_decay_k<T><<<nblocks(rows * H * dim, 256), 256, 0, s>>>(
                    (const T*)z, ld_z, bias, a_log, out, rows, H, dim)));
   return (int)hipGetLastError();

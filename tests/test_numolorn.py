@@ -1250,3 +1250,40 @@ def test_router_and_pair_hash_kernels_against_eager(E, top, count, keep,
     assert (res[0][1] - res[1][1]).abs().max().item() < 1e-5
     assert torch.equal(res[0][2], res[1][2])
     assert torch.equal(res[0][3], res[1][3])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,v,gated", [(4, 32, True), (3, 6, True),
+                                       (16, 128, False), (5, 20, False)])
+def test_head_merge_kernel_against_eager(H, v, gated, dtype, monkeypatch):
+    from deepspeed_amd.ops.latent_attention import gate_merge_heads
+    g = torch.Generator().manual_seed(H * v)
+    o = torch.randn(H, 37, v, generator=g).to(DEV, dtype)
+    gate = torch.rand(37, H, generator=g).to(DEV) if gated else None
+    got = gate_merge_heads(o, gate).float()
+    monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+    want = gate_merge_heads(o, gate).float()
+    assert got.shape == (37, H * v)
+    assert (got - want).abs().max().item() < \
+        (1e-6 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,d,skip", [(6, 64, 0), (6, 64, 8), (3, 20, 0),
+                                      (4, 128, 3)])
+def test_decay_kernel_on_slices_against_eager(H, d, skip, dtype, monkeypatch):
+    """Eight channels per thread where width, stride and address allow it,
+    one otherwise (a slice that starts 3 columns in)."""
+    from deepspeed_amd.ops.linear_recurrence import softplus_decay
+    g = torch.Generator().manual_seed(H * d + skip)
+    wide = (2 * torch.randn(29, H * d + 16, generator=g)).to(DEV, dtype)
+    bias = torch.randn(H * d, generator=g).to(DEV)
+    a_log = (torch.randn(H, generator=g) - 1).to(DEV)
+    z = wide[:, skip:skip + H * d]
+    got = softplus_decay(z, bias, a_log, H)
+    monkeypatch.setenv("DS_AMD_SERVING_EAGER", "1")
+    want = softplus_decay(z, bias, a_log, H)
+    assert got.shape == (29, H, d) and got.dtype == torch.float32
+    assert (got - want).abs().max().item() < 2e-6
