@@ -547,12 +547,22 @@ class NumolornForCausalLM(nn.Module):
                 taps.append(x.clone())
         if pending is not None:
             scaled_add_(x, *pending)
-        # logits = table . (norm(x) * w) * scale: the scale rides on the
-        # norm's weight, so no pass over [rows, vocab] is needed for it
+        return F.linear(rms_norm_rows(x, self._final_weight(), eps, dt, rows),
+                        self.embed)
+
+    def _final_weight(self):
+        """logits = table . (norm(x) * w) * scale: the scale rides on the
+        norm's weight, so no pass over [rows, vocab] is needed for it. The
+        product is kept until the weight changes."""
         w = self.final_norm
-        if self.cfg.logit_scale != 1.0:
-            w = w * self.cfg.logit_scale
-        return F.linear(rms_norm_rows(x, w, eps, dt, rows), self.embed)
+        if self.cfg.logit_scale == 1.0:
+            return w
+        kept = self.__dict__.get("_scaled_final")
+        if kept is None or kept[0] != (w._version, w.device, w.data_ptr()):
+            kept = ((w._version, w.device, w.data_ptr()),
+                    w.detach() * self.cfg.logit_scale)
+            self.__dict__["_scaled_final"] = kept
+        return kept[1]
 
     def num_parameters(self):
         return sum(p.numel() for p in self.parameters())

@@ -216,7 +216,7 @@ class RoutedExperts(nn.Module):
                 # after the experts' results: block number ``experts``
                 y = torch.cat([y, h], 0)
                 idx = idx.clamp(max=self.experts)
-            inv = idx * T + torch.arange(T, device=h.device)[:, None]
+            inv = torch.add(self._token_ids(T, h.device), idx, alpha=T)
         else:
             y, inv = self._grouped(h, idx)
         sh = sg = None
@@ -226,6 +226,16 @@ class RoutedExperts(nn.Module):
         return moe_combine(y, inv, weight, sh, sg)
 
     DENSE_MAX_PICKS = 64
+
+    def _token_ids(self, T, device):
+        """[T, 1] int64 0..T-1, kept per step size (decode steps repeat)."""
+        cache = self.__dict__.setdefault("_ids", {})
+        key = (T, str(device))
+        if key not in cache:
+            if len(cache) > 64:
+                cache.clear()
+            cache[key] = torch.arange(T, device=device)[:, None]
+        return cache[key]
 
     def _grouped(self, h, idx):
         """Tokens sorted by expert; one pair of GEMMs per expert that has
